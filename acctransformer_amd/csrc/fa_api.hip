@@ -1,0 +1,211 @@
+// C ABI of the gfx950 attention kernels: argument validation, workspace
+// carving, kernel selection.  Declared in include/acct_fa.h.
+#include <hip/hip_runtime.h>
+#include <atomic>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "../../include/acct_fa.h"
+#include "fa_common.hpp"
+#include "fa_launch.hpp"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_dev_state[kMaxDevices];   // 0 unknown, 1 gfx950, 2 other
+std::atomic<int> g_dev_cus[kMaxDevices];
+
+int check_device(int* n_cu) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(ACCT_E_ARCH, "no HIP device is current");
+  if (dev < 0 || dev >= kMaxDevices) return fail(ACCT_E_ARCH, "device ordinal %d out of range", dev);
+  int st = g_dev_state[dev].load(std::memory_order_acquire);
+  if (st == 0) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return fail(ACCT_E_ARCH, "hipGetDeviceProperties failed");
+    g_dev_cus[dev].store(prop.multiProcessorCount, std::memory_order_relaxed);
+    st = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 2;
+    g_dev_state[dev].store(st, std::memory_order_release);
+  }
+  if (st != 1) return fail(ACCT_E_ARCH, "device %d is not gfx950; this library carries gfx950 code only", dev);
+  *n_cu = g_dev_cus[dev].load(std::memory_order_relaxed);
+  return ACCT_OK;
+}
+
+size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+bool strides_zero(const int64_t s[3]) { return s[0] == 0 && s[1] == 0 && s[2] == 0; }
+
+// Checks that need no device: used by the entry points and by the workspace queries.
+int validate(const acct_fa_params* p) {
+  if (!p) return fail(ACCT_E_NULLPTR, "params is NULL");
+  if (p->dtype != ACCT_F16 && p->dtype != ACCT_BF16) return fail(ACCT_E_DTYPE, "dtype %d is neither ACCT_F16 nor ACCT_BF16", p->dtype);
+  if (p->B <= 0 || p->N <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->D <= 0)
+    return fail(ACCT_E_SHAPE, "extents must be positive: B=%d N=%d Sq=%d Sk=%d D=%d", p->B, p->N, p->Sq, p->Sk, p->D);
+  if (p->D > 256) return fail(ACCT_E_HEADDIM, "head_dim too large, reduce head_dim and try again. (D=%d > 256)", p->D);
+  if (p->D != 64 && p->D != 80 && p->D != 128) return fail(ACCT_E_HEADDIM, "head_dim %d not built; supported: 64, 80, 128", p->D);
+  if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return fail(ACCT_E_PARAM, "scale must be positive and finite, got %g", (double)p->scale);
+  if (!(p->keep_prob > 0.f && p->keep_prob <= 1.f)) return fail(ACCT_E_PARAM, "keep_prob must be in (0, 1], got %g", (double)p->keep_prob);
+  if (p->prev_block_num < 0 || p->next_block_num < 0) return fail(ACCT_E_PARAM, "prev_block_num / next_block_num must be >= 0");
+  switch (p->mask_kind) {
+    case ACCT_MASK_NONE: case ACCT_MASK_CAUSAL: break;
+    case ACCT_MASK_DENSE_U8: case ACCT_MASK_TILE_U8:
+      if (!p->attn_mask) return fail(ACCT_E_NULLPTR, "attn_mask is NULL but mask_kind=%d needs a tensor", p->mask_kind);
+      break;
+    default: return fail(ACCT_E_PARAM, "unknown mask_kind %d", p->mask_kind);
+  }
+  if (p->mask_stride_b < 0 || (p->mask_kind == ACCT_MASK_DENSE_U8 && p->mask_stride_b != 0 && p->mask_stride_b < (int64_t)p->Sq * p->Sk))
+    return fail(ACCT_E_SHAPE, "mask_stride_b must be 0 (broadcast) or >= Sq*Sk");
+  if (!p->q || !p->k || !p->v) return fail(ACCT_E_NULLPTR, "q, k and v must be non-NULL");
+  const int64_t* st[4] = {p->q_stride, p->k_stride, p->v_stride, p->o_stride};
+  const void* ptrs[3] = {p->q, p->k, p->v};
+  for (int i = 0; i < 4; i++) {
+    if (strides_zero(st[i])) continue;
+    for (int j = 0; j < 3; j++)
+      if (st[i][j] < 0 || st[i][j] % 8 != 0) return fail(ACCT_E_SHAPE, "strides must be non-negative multiples of 8 elements");
+    if (st[i][2] < p->D) return fail(ACCT_E_SHAPE, "row stride smaller than D");
+  }
+  for (int i = 0; i < 3; i++)
+    if ((uintptr_t)ptrs[i] & 15) return fail(ACCT_E_SHAPE, "q, k and v must be 16-byte aligned");
+  if (p->alibi && (p->alibi_stride_b < 0 || p->alibi_stride_h < 0 || p->alibi_stride_q < 0))
+    return fail(ACCT_E_SHAPE, "alibi strides must be >= 0");
+  return ACCT_OK;
+}
+
+void fill_strides(const int64_t s[3], int N, int S, int D, int64_t* sb, int64_t* sh, int64_t* ss) {
+  if (strides_zero(s)) { *ss = D; *sh = (int64_t)S * D; *sb = (int64_t)N * S * D; }
+  else { *sb = s[0]; *sh = s[1]; *ss = s[2]; }
+}
+
+acct::FaArgs make_args(const acct_fa_params* p) {
+  acct::FaArgs a;
+  memset(&a, 0, sizeof(a));
+  a.q = p->q; a.k = p->k; a.v = p->v;
+  a.mask = (p->mask_kind == ACCT_MASK_DENSE_U8 || p->mask_kind == ACCT_MASK_TILE_U8) ? p->attn_mask : nullptr;
+  a.drop = p->keep_prob < 1.f || p->drop_mask ? p->drop_mask : nullptr;
+  a.alibi = p->alibi;
+  a.B = p->B; a.N = p->N; a.Sq = p->Sq; a.Sk = p->Sk;
+  a.Tr = (p->Sq + 127) / 128; a.Tc = (p->Sk + 127) / 128;
+  fill_strides(p->q_stride, p->N, p->Sq, p->D, &a.q_sb, &a.q_sh, &a.q_ss);
+  fill_strides(p->k_stride, p->N, p->Sk, p->D, &a.k_sb, &a.k_sh, &a.k_ss);
+  fill_strides(p->v_stride, p->N, p->Sk, p->D, &a.v_sb, &a.v_sh, &a.v_ss);
+  fill_strides(p->o_stride, p->N, p->Sq, p->D, &a.o_sb, &a.o_sh, &a.o_ss);
+  a.mask_sb = p->mask_kind == ACCT_MASK_DENSE_U8 ? p->mask_stride_b : 0;
+  a.al_sb = p->alibi_stride_b; a.al_sh = p->alibi_stride_h; a.al_sq = p->alibi_stride_q;
+  a.scale = p->scale;
+  a.scale_log2e = p->scale * acct::kLog2e;
+  a.inv_keep = 1.0f / p->keep_prob;
+  a.mask_add_raw = acct::kMaskFill / p->scale;
+  a.prev_blk = p->prev_block_num > ACCT_BLOCK_UNBOUNDED ? ACCT_BLOCK_UNBOUNDED : p->prev_block_num;
+  a.next_blk = p->next_block_num > ACCT_BLOCK_UNBOUNDED ? ACCT_BLOCK_UNBOUNDED : p->next_block_num;
+  a.mask_kind = p->mask_kind;
+  return a;
+}
+
+bool is_general(const acct_fa_params* p) {
+  return p->mask_kind == ACCT_MASK_DENSE_U8 || p->mask_kind == ACCT_MASK_TILE_U8 || p->drop_mask || p->alibi;
+}
+
+size_t flag_bytes(const acct_fa_params* p) {
+  if (p->mask_kind != ACCT_MASK_DENSE_U8) return 0;
+  const size_t MB = p->mask_stride_b ? p->B : 1;
+  return align_up(MB * (size_t)((p->Sq + 127) / 128) * (size_t)((p->Sk + 127) / 128), 256);
+}
+
+int env_int(const char* name, int dflt) {
+  const char* s = getenv(name);
+  return s && *s ? atoi(s) : dflt;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* acct_last_error(void) { return g_err; }
+int acct_version(void) { return ACCT_FA_VERSION; }
+
+size_t acct_fa_fwd_workspace_bytes(const acct_fa_params* p) {
+  if (!p) return 0;
+  return flag_bytes(p);
+}
+
+size_t acct_fa_bwd_workspace_bytes(const acct_fa_params* p) {
+  if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0) return 0;
+  return align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + flag_bytes(p);
+}
+
+int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, size_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  int rc = validate(p);
+  if (rc) return rc;
+  if (!O || !LSE) return fail(ACCT_E_NULLPTR, "O and LSE must be non-NULL");
+  if ((uintptr_t)O & 7) return fail(ACCT_E_SHAPE, "O must be 8-byte aligned");
+  if (p->keep_prob < 1.f && !p->drop_mask) return fail(ACCT_E_NULLPTR, "keep_prob < 1 needs a drop_mask");
+  const size_t need = acct_fa_fwd_workspace_bytes(p);
+  if (need && (!workspace || workspace_bytes < need))
+    return fail(ACCT_E_WORKSPACE, "forward workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
+  int n_cu = 0;
+  rc = check_device(&n_cu);
+  if (rc) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  acct::FaArgs a = make_args(p);
+  a.o = O; a.lse = LSE;
+  if (p->mask_kind == ACCT_MASK_DENSE_U8) {
+    a.blkflags = (const uint8_t*)workspace;
+    hipError_t e = acct::launch_mask_blocks(a, (uint8_t*)workspace, p->mask_stride_b ? p->B : 1, st);
+    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
+  }
+  // 64 query rows per wave (256 per workgroup) once that still fills the chip
+  int qg = ((long long)p->B * p->N * ((p->Sq + 255) / 256) >= n_cu) ? 2 : 1;
+  qg = env_int("ACCT_FA_FWD_QG", qg) == 1 ? 1 : 2;
+  hipError_t e = acct::launch_fwd(a, p->dtype, p->D, is_general(p), qg, st);
+  if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "forward kernel: %s", hipGetErrorString(e));
+  return ACCT_OK;
+}
+
+int acct_fa_bwd(const acct_fa_params* p, const void* O, const void* dO, const float* LSE, void* dQ, void* dK, void* dV,
+                void* workspace, size_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  int rc = validate(p);
+  if (rc) return rc;
+  if (!O || !dO || !LSE || !dQ || !dK || !dV) return fail(ACCT_E_NULLPTR, "O, dO, LSE, dQ, dK and dV must be non-NULL");
+  if (((uintptr_t)O | (uintptr_t)dO | (uintptr_t)dQ | (uintptr_t)dK | (uintptr_t)dV) & 15)
+    return fail(ACCT_E_SHAPE, "O, dO, dQ, dK and dV must be 16-byte aligned");
+  if (p->keep_prob < 1.f && !p->drop_mask) return fail(ACCT_E_NULLPTR, "keep_prob < 1 needs a drop_mask");
+  const size_t need = acct_fa_bwd_workspace_bytes(p);
+  if (!workspace || workspace_bytes < need)
+    return fail(ACCT_E_WORKSPACE, "backward workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
+  if ((uintptr_t)workspace & 255) return fail(ACCT_E_WORKSPACE, "workspace must be 256-byte aligned");
+  int n_cu = 0;
+  rc = check_device(&n_cu);
+  if (rc) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  acct::FaArgs a = make_args(p);
+  a.o = const_cast<void*>(O); a.lse = const_cast<float*>(LSE);
+  a.dout = dO; a.dq = dQ; a.dk = dK; a.dv = dV;
+  a.delta = (float*)workspace;
+  if (p->mask_kind == ACCT_MASK_DENSE_U8) {
+    uint8_t* flags = (uint8_t*)workspace + align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256);
+    a.blkflags = flags;
+    hipError_t e = acct::launch_mask_blocks(a, flags, p->mask_stride_b ? p->B : 1, st);
+    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
+  }
+  hipError_t e = acct::launch_bwd(a, p->dtype, p->D, is_general(p), st);
+  if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "backward kernels: %s", hipGetErrorString(e));
+  return ACCT_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,133 @@
+// Device-side building blocks shared by the gfx950 attention kernels:
+// vector types, the 32x32x16 MFMA wrappers, LDS fragment reads and the
+// kernel argument block.  CDNA4 only (wave64, MFMA, ds_read_*_tr_b16).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace acct {
+
+typedef _Float16 f16;
+typedef __bf16 bf16;
+typedef f16 f16x8 __attribute__((ext_vector_type(8)));
+typedef f16 f16x4 __attribute__((ext_vector_type(4)));
+typedef f16 f16x2 __attribute__((ext_vector_type(2)));
+typedef bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+#define ACCT_LDS __attribute__((address_space(3)))
+#define ACCT_DEV __device__ __forceinline__
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kMaskFill = -10000.0f;   // additive mask value of the reference (constants.py:24)
+
+// ---- element-type traits ---------------------------------------------------
+template <typename T> struct Elem;
+template <> struct Elem<f16> {
+  using V8 = f16x8; using V4 = f16x4; using V2 = f16x2;
+  static ACCT_DEV f32x16 mfma(V8 a, V8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+  static ACCT_DEV V2 cvt2(float x, float y) { f32x2 t = {x, y}; return __builtin_convertvector(t, V2); }
+};
+template <> struct Elem<bf16> {
+  using V8 = bf16x8; using V4 = bf16x4; using V2 = bf16x2;
+  static ACCT_DEV f32x16 mfma(V8 a, V8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+  static ACCT_DEV V2 cvt2(float x, float y) { f32x2 t = {x, y}; return __builtin_convertvector(t, V2); }
+};
+
+// The MFMA 32x32x16 register layouts used throughout (lane l, g = l / 32):
+//   A (32 x 16): lane holds row  l % 32, k = 8g .. 8g+7
+//   B (16 x 32): lane holds col  l % 32, k = 8g .. 8g+7
+//   C (32 x 32): lane holds col  l % 32, rows 8*(r/4) + 4g + r%4 for r = 0..15
+// A C tile can therefore be fed back as a B operand of a product that
+// contracts over C's rows: registers 8h..8h+7 are the k = 8g..8g+7 slots of
+// k-step h, i.e. rows 16h + 8*(e/4) + 4g + e%4 (e = 0..7) of the C tile.
+
+// 16-byte LDS read of an A/B fragment stored row-major.
+template <typename T>
+ACCT_DEV typename Elem<T>::V8 lds_read_frag(const ACCT_LDS char* p) {
+  return *reinterpret_cast<const ACCT_LDS typename Elem<T>::V8*>(p);
+}
+
+// Transposed LDS read (ds_read_b64_tr_b16).  Within each block of 16 lanes,
+// lane i supplies the address of 4 consecutive 16-bit elements
+// M[k0 + i/4][n0 + 4*(i%4) ..]; lane j receives M[k0 + 0..3][n0 + j].
+ACCT_DEV i16x4 lds_read_tr(const ACCT_LDS char* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((ACCT_LDS i16x4*)(p));
+}
+
+template <typename T>
+ACCT_DEV typename Elem<T>::V8 join_tr(i16x4 lo, i16x4 hi) {
+  typedef short i16x8 __attribute__((ext_vector_type(8)));
+  i16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(typename Elem<T>::V8, v);
+}
+
+// reductions over the lane pair (l, l ^ 32): v_permlane32_swap leaves the low
+// halves of both operands in one register and the high halves in the other.
+ACCT_DEV float pair_max(float x) {
+  u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+ACCT_DEV float pair_sum(float x) {
+  u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+ACCT_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ---- kernel arguments --------------------------------------------------------
+struct FaArgs {
+  const void* q; const void* k; const void* v;
+  void* o; float* lse;                 // fwd outputs / bwd inputs
+  const void* dout; void* dq; void* dk; void* dv; float* delta;   // bwd only
+  const uint8_t* mask; const uint8_t* drop; const void* alibi;
+  const uint8_t* blkflags;             // [MB, Tr, Tc] block classes of a dense mask
+  int B, N, Sq, Sk;
+  int Tr, Tc;                          // number of 128-row / 128-column blocks
+  int64_t q_sb, q_sh, q_ss;
+  int64_t k_sb, k_sh, k_ss;
+  int64_t v_sb, v_sh, v_ss;
+  int64_t o_sb, o_sh, o_ss;
+  int64_t mask_sb;
+  int64_t al_sb, al_sh, al_sq;
+  float scale, scale_log2e, inv_keep;
+  float mask_add_raw;                  // -10000 / scale: the mask in raw q.k units
+  int prev_blk, next_blk;
+  int mask_kind;
+  int n_tiles;                         // tiles along the owner dimension
+};
+
+enum : int { kMaskNone = 0, kMaskDense = 1, kMaskTile = 3, kMaskCausal = 4 };
+enum : uint8_t { kBlkClean = 0, kBlkApply = 1, kBlkSkip = 2 };
+
+// four consecutive mask / dropout bytes starting at column kv of a row
+ACCT_DEV uint32_t load_u8x4(const uint8_t* row, int kv, int limit, bool vec_ok) {
+  if (vec_ok && kv + 4 <= limit) return *reinterpret_cast<const uint32_t*>(row + kv);
+  uint32_t r = 0;
+#pragma unroll
+  for (int e = 0; e < 4; e++)
+    if (kv + e < limit) r |= (uint32_t)row[kv + e] << (8 * e);
+  return r;
+}
+
+template <typename T>
+ACCT_DEV void load_bias4(const T* row, int kv, int limit, bool vec_ok, float out[4]) {
+  if (vec_ok && kv + 4 <= limit) {
+    typename Elem<T>::V4 t = *reinterpret_cast<const typename Elem<T>::V4*>(row + kv);
+#pragma unroll
+    for (int e = 0; e < 4; e++) out[e] = (float)t[e];
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; e++) out[e] = (kv + e < limit) ? (float)row[kv + e] : 0.f;
+  }
+}
+
+}  // namespace acct

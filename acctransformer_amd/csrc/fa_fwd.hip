@@ -1,0 +1,347 @@
+// FlashAttention2 forward for gfx950 (CDNA4).
+//
+// Replaces the reference's forward kernel builder
+// (train/acctransformer/flash_attention/ops/flash_attention/flash_attention_fwd.py:308-474:
+// Q-outer / KV-inner loops, online softmax, O rescale, O/l and L = m + ln l).
+//
+// Work split: one workgroup (4 waves) owns 128*QG query rows of one (batch,
+// head); each wave owns 32*QG of them.  K and V tiles of 64 rows are staged
+// through LDS (double buffered) and shared by the 4 waves.  The wave computes
+// the TRANSPOSED score tile S^T = K Q^T with 32x32x16 MFMAs, so every lane
+// holds scores of a single query row (column l%32 of the MFMA C tile): the
+// online-softmax state (running max, running sum) is per lane, row
+// reductions are in-register plus one swap with lane l^32, and the C tile is
+// directly the B operand of O^T += V^T P^T.  V^T fragments come from the
+// row-major V tile through transposed LDS reads.
+#include "fa_common.hpp"
+#include "fa_launch.hpp"
+
+namespace acct {
+
+template <int D> struct FwdCfg {
+  static constexpr int KS = D / 16;             // k-steps of K Q^T
+  static constexpr int DB = (D + 31) / 32;      // 32-row blocks of O^T
+  static constexpr int DP = DB * 32;
+  static constexpr int CPR = D / 8;             // 16-byte chunks per row
+  static constexpr int ROWB = DP * 2 + 16;      // LDS row pitch (bytes): +16 keeps b128 reads conflict free
+  static constexpr int BN = 64;                 // kv rows per tile
+  static constexpr int TILEB = BN * ROWB;
+  static constexpr int NLD = (BN * CPR + 255) / 256;
+};
+
+template <typename T, int D>
+ACCT_DEV void tile_load(const T* base, int64_t row_stride, int row0, int nrows, u32x4 (&reg)[FwdCfg<D>::NLD]) {
+  using C = FwdCfg<D>;
+#pragma unroll
+  for (int i = 0; i < C::NLD; i++) {
+    const int idx = threadIdx.x + 256 * i;
+    const int row = idx / C::CPR, ch = idx % C::CPR;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (idx < C::BN * C::CPR && row0 + row < nrows)
+      v = *reinterpret_cast<const u32x4*>(base + (int64_t)(row0 + row) * row_stride + ch * 8);
+    reg[i] = v;
+  }
+}
+
+template <int D>
+ACCT_DEV void tile_store(ACCT_LDS char* buf, const u32x4 (&reg)[FwdCfg<D>::NLD]) {
+  using C = FwdCfg<D>;
+#pragma unroll
+  for (int i = 0; i < C::NLD; i++) {
+    const int idx = threadIdx.x + 256 * i;
+    const int row = idx / C::CPR, ch = idx % C::CPR;
+    if (idx < C::BN * C::CPR) *reinterpret_cast<ACCT_LDS u32x4*>(buf + row * C::ROWB + ch * 16) = reg[i];
+  }
+}
+
+template <typename T, int D, int QG, bool GENERAL>
+__global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
+  using E = Elem<T>;
+  using V8 = typename E::V8;
+  using C = FwdCfg<D>;
+  constexpr int BM = 128 * QG;
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 buffers][K tile | V tile]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, g = lane >> 5;
+  const int BH = a.B * a.N;
+  const int bh = blockIdx.x % BH;
+  const int qt = a.n_tiles - 1 - (int)(blockIdx.x / BH);   // heaviest (latest) causal tiles first
+  const int b = bh / a.N, h = bh % a.N;
+  const int q0 = qt * BM;
+  const int wq0 = q0 + wave * 32 * QG;                      // first query row of this wave
+  const int q_end = min(q0 + BM, a.Sq);                     // one past the last valid row of the block
+  const int wq_end = min(wq0 + 32 * QG, a.Sq);
+
+  const T* qp = (const T*)a.q + b * a.q_sb + h * a.q_sh;
+  const T* kp = (const T*)a.k + b * a.k_sb + h * a.k_sh;
+  const T* vp = (const T*)a.v + b * a.v_sb + h * a.v_sh;
+
+  // ---- visible kv tiles of this block (128-block band; causal clips the top) ----
+  const int qb_lo = q0 / 128, qb_hi = (q_end - 1) / 128;
+  const int kvb_lo = max(0, qb_lo - a.prev_blk), kvb_hi = min(a.Tc - 1, qb_hi + a.next_blk);
+  int j_lo = kvb_lo * 2, j_hi = min(kvb_hi * 2 + 1, (a.Sk - 1) / 64);
+  const bool causal = a.mask_kind == kMaskCausal;
+  if (causal) j_hi = min(j_hi, (q_end - 1) / 64);
+  const int wqb = wq0 / 128;                                // 128-block of this wave's rows
+
+  // ---- Q fragments (B operand of K Q^T): lane holds row l32, d = 16t + 8g .. +7 ----
+  V8 qf[QG][C::KS];
+#pragma unroll
+  for (int gq = 0; gq < QG; gq++) {
+    const int row = wq0 + 32 * gq + l32;
+#pragma unroll
+    for (int t = 0; t < C::KS; t++) {
+      V8 z = {};
+      qf[gq][t] = (row < a.Sq) ? *reinterpret_cast<const V8*>(qp + (int64_t)row * a.q_ss + 16 * t + 8 * g) : z;
+    }
+  }
+
+  f32x16 o[QG][C::DB];
+  float m[QG], lsum[QG];
+#pragma unroll
+  for (int gq = 0; gq < QG; gq++) {
+    m[gq] = -INFINITY;
+    lsum[gq] = 0.f;
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) o[gq][db][r] = 0.f;
+  }
+
+  const float cmul = GENERAL ? 1.0f : a.scale_log2e;   // exp2 argument = s * cmul - m * cmul
+  const int mb = a.mask_sb ? b : 0;
+  const uint8_t* maskp = GENERAL && a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
+  const uint8_t* dropp = GENERAL && a.drop ? a.drop + ((int64_t)bh * a.Sq) * a.Sk : nullptr;
+  const T* alibip = GENERAL && a.alibi ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
+  const bool mask_vec = GENERAL && (a.mask_kind == kMaskDense ? (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0
+                                                              : ((uintptr_t)a.mask & 3) == 0);
+  const bool drop_vec = GENERAL && (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 3) == 0;
+  const bool alibi_vec = GENERAL && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
+
+  if (j_lo <= j_hi) {
+    u32x4 kreg[C::NLD], vreg[C::NLD];
+    tile_load<T, D>(kp, a.k_ss, j_lo * 64, a.Sk, kreg);
+    tile_load<T, D>(vp, a.v_ss, j_lo * 64, a.Sk, vreg);
+    tile_store<D>(smem, kreg);
+    tile_store<D>(smem + C::TILEB, vreg);
+    __syncthreads();
+
+    for (int j = j_lo; j <= j_hi; j++) {
+      const int buf = (j - j_lo) & 1;
+      ACCT_LDS char* kbuf = smem + buf * 2 * C::TILEB;
+      ACCT_LDS char* vbuf = kbuf + C::TILEB;
+      const bool more = j < j_hi;
+      if (more) {
+        tile_load<T, D>(kp, a.k_ss, (j + 1) * 64, a.Sk, kreg);
+        tile_load<T, D>(vp, a.v_ss, (j + 1) * 64, a.Sk, vreg);
+      }
+      const int kv0 = j * 64;
+      const int kvb = j >> 1;
+      bool act = (kvb - a.next_blk <= wqb) && (wqb <= kvb + a.prev_blk) && (wq0 < a.Sq);
+      if (causal) act = act && (kv0 <= wq_end - 1);
+      bool apply_mask = false;
+      if (GENERAL) {
+        if (a.mask_kind == kMaskDense && act) {
+          const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + wqb) * a.Tc + kvb];
+          act = f != kBlkSkip;
+          apply_mask = f == kBlkApply;
+        } else if (a.mask_kind == kMaskTile) {
+          apply_mask = wqb == kvb;
+        }
+      }
+      if (act) {
+        // ---- S^T = K Q^T : s[gq][c] is the 32(kv) x 32(q) tile of kv chunk c ----
+        f32x16 s[QG][2];
+#pragma unroll
+        for (int gq = 0; gq < QG; gq++)
+#pragma unroll
+          for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[gq][c][r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < C::KS; t++) {
+#pragma unroll
+          for (int c = 0; c < 2; c++) {
+            const V8 kf = lds_read_frag<T>(kbuf + (32 * c + l32) * C::ROWB + (16 * t + 8 * g) * 2);
+#pragma unroll
+            for (int gq = 0; gq < QG; gq++) s[gq][c] = E::mfma(kf, qf[gq][t], s[gq][c]);
+          }
+        }
+        // element (gq, c, r): q = wq0 + 32 gq + l32 ; kv = kv0 + 32 c + 8 (r/4) + 4 g + r%4
+        const bool tail = kv0 + 64 > a.Sk;
+        const bool diag = causal && (kv0 + 63 > wq0);
+        typename E::V8 pf[QG][2][2];
+#pragma unroll
+        for (int gq = 0; gq < QG; gq++) {
+          const int qrow = wq0 + 32 * gq + l32;
+          const int qrow_c = min(qrow, a.Sq - 1);            // clamped for side-input addressing
+          if (GENERAL) {
+#pragma unroll
+            for (int c = 0; c < 2; c++)
+#pragma unroll
+              for (int r4 = 0; r4 < 4; r4++) {
+                const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
+                float bias[4] = {0.f, 0.f, 0.f, 0.f};
+                if (alibip) load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
+                uint32_t mbits = 0;
+                if (apply_mask) {
+                  if (a.mask_kind == kMaskDense) mbits = load_u8x4(maskp + (int64_t)qrow_c * a.Sk, kv, a.Sk, mask_vec);
+                  else mbits = load_u8x4(maskp + (qrow_c & 127) * 128, kv & 127, 128, mask_vec);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                  float x = s[gq][c][4 * r4 + e] * a.scale_log2e + bias[e] * kLog2e;
+                  if ((mbits >> (8 * e)) & 0xffu) x += kMaskFill * kLog2e;
+                  if (causal && kv + e > qrow) x += kMaskFill * kLog2e;
+                  if (kv + e >= a.Sk) x = -INFINITY;
+                  s[gq][c][4 * r4 + e] = x;
+                }
+              }
+          } else {
+            if (diag || tail) {
+#pragma unroll
+              for (int c = 0; c < 2; c++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                  const int kv = kv0 + 32 * c + 8 * (r >> 2) + 4 * g + (r & 3);
+                  float x = s[gq][c][r];
+                  if (causal && kv > qrow) x += a.mask_add_raw;
+                  if (kv >= a.Sk) x = -INFINITY;
+                  s[gq][c][r] = x;
+                }
+            }
+          }
+          // ---- online softmax for query row qrow ----
+          float mx = s[gq][0][0];
+#pragma unroll
+          for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[gq][c][r]);
+          mx = pair_max(mx);
+          const float m_new = fmaxf(m[gq], mx);
+          const float alpha = fast_exp2((m[gq] - m_new) * cmul);
+          const float mc = m_new * cmul;
+          m[gq] = m_new;
+          float rs = 0.f;
+          float p[2][16];
+#pragma unroll
+          for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+              p[c][r] = fast_exp2(__builtin_fmaf(s[gq][c][r], cmul, -mc));
+              rs += p[c][r];
+            }
+          lsum[gq] = lsum[gq] * alpha + rs;                  // row sum BEFORE dropout
+          if (GENERAL && dropp) {
+#pragma unroll
+            for (int c = 0; c < 2; c++)
+#pragma unroll
+              for (int r4 = 0; r4 < 4; r4++) {
+                const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
+                const uint32_t dbits = load_u8x4(dropp + (int64_t)qrow_c * a.Sk, kv, a.Sk, drop_vec);
+#pragma unroll
+                for (int e = 0; e < 4; e++) p[c][4 * r4 + e] *= ((dbits >> (8 * e)) & 0xffu) ? a.inv_keep : 0.f;
+              }
+          }
+#pragma unroll
+          for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) {
+              typename E::V2 t0 = E::cvt2(p[c][8 * hh + 0], p[c][8 * hh + 1]);
+              typename E::V2 t1 = E::cvt2(p[c][8 * hh + 2], p[c][8 * hh + 3]);
+              typename E::V2 t2 = E::cvt2(p[c][8 * hh + 4], p[c][8 * hh + 5]);
+              typename E::V2 t3 = E::cvt2(p[c][8 * hh + 6], p[c][8 * hh + 7]);
+              V8 pv = {t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+              pf[gq][c][hh] = pv;
+            }
+          if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int db = 0; db < C::DB; db++)
+#pragma unroll
+              for (int r = 0; r < 16; r++) o[gq][db][r] *= alpha;
+          }
+        }
+        // ---- O^T += V^T P^T ----
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+          for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+            for (int db = 0; db < C::DB; db++) {
+              const ACCT_LDS char* vaddr = vbuf + (32 * c + 16 * hh + 4 * g + ((lane & 15) >> 2)) * C::ROWB +
+                                           (32 * db + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+              const V8 vf = join_tr<T>(lds_read_tr(vaddr), lds_read_tr(vaddr + 8 * C::ROWB));
+#pragma unroll
+              for (int gq = 0; gq < QG; gq++) o[gq][db] = E::mfma(vf, pf[gq][c][hh], o[gq][db]);
+            }
+      }
+      if (more) {
+        ACCT_LDS char* nk = smem + (buf ^ 1) * 2 * C::TILEB;
+        tile_store<D>(nk, kreg);
+        tile_store<D>(nk + C::TILEB, vreg);
+      }
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue: O = O^T / l, LSE = m + ln l ----
+  T* op = (T*)a.o + b * a.o_sb + h * a.o_sh;
+  const float mnat = GENERAL ? kLn2 : a.scale;
+#pragma unroll
+  for (int gq = 0; gq < QG; gq++) {
+    const int row = wq0 + 32 * gq + l32;
+    const float l = pair_sum(lsum[gq]);
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    if (row < a.Sq) {
+      if (g == 0) a.lse[(int64_t)bh * a.Sq + row] = l > 0.f ? m[gq] * mnat + __logf(l) : -INFINITY;
+#pragma unroll
+      for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; r4++) {
+          const int d = 32 * db + 8 * r4 + 4 * g;
+          if (d < D) {
+            typename E::V2 t0 = E::cvt2(o[gq][db][4 * r4 + 0] * inv, o[gq][db][4 * r4 + 1] * inv);
+            typename E::V2 t1 = E::cvt2(o[gq][db][4 * r4 + 2] * inv, o[gq][db][4 * r4 + 3] * inv);
+            typename E::V4 ov = {t0[0], t0[1], t1[0], t1[1]};
+            *reinterpret_cast<typename E::V4*>(op + (int64_t)row * a.o_ss + d) = ov;
+          }
+        }
+    }
+  }
+}
+
+template <typename T, int D, int QG, bool GENERAL>
+static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
+  using C = FwdCfg<D>;
+  constexpr int BM = 128 * QG;
+  a.n_tiles = (a.Sq + BM - 1) / BM;
+  const size_t smem = 4 * (size_t)C::TILEB;
+  auto kern = fa_fwd_kernel<T, D, QG, GENERAL>;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  if (e != hipSuccess) return e;
+  const long long nblk = (long long)a.n_tiles * a.B * a.N;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(256), smem, st, a);
+  return hipGetLastError();
+}
+
+template <typename T, int D>
+static hipError_t launch_fwd_d(const FaArgs& a, bool general, int qg, hipStream_t st) {
+  if (general) return qg == 2 ? launch_fwd_t<T, D, 2, true>(a, st) : launch_fwd_t<T, D, 1, true>(a, st);
+  return qg == 2 ? launch_fwd_t<T, D, 2, false>(a, st) : launch_fwd_t<T, D, 1, false>(a, st);
+}
+
+hipError_t launch_fwd(const FaArgs& a, int dtype, int D, bool general, int qg, hipStream_t st) {
+  if (dtype == 0) {
+    if (D == 128) return launch_fwd_d<f16, 128>(a, general, qg, st);
+    if (D == 64) return launch_fwd_d<f16, 64>(a, general, qg, st);
+    if (D == 80) return launch_fwd_d<f16, 80>(a, general, qg, st);
+  } else {
+    if (D == 128) return launch_fwd_d<bf16, 128>(a, general, qg, st);
+    if (D == 64) return launch_fwd_d<bf16, 64>(a, general, qg, st);
+    if (D == 80) return launch_fwd_d<bf16, 80>(a, general, qg, st);
+  }
+  return hipErrorInvalidValue;
+}
+
+}  // namespace acct

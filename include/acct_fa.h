@@ -1,0 +1,120 @@
+/*
+ * acct_fa.h -- C ABI of the MI355X (gfx950) FlashAttention2 / TriangleAttention
+ * hot path.  Plain pointers and sizes only; every pointer is a DEVICE pointer
+ * unless a comment says otherwise; the caller owns every buffer; the library
+ * never allocates, never throws, never synchronises: each call enqueues its
+ * kernels on `stream` (a hipStream_t passed as void*; NULL = default stream).
+ *
+ * Citations are file:line in the reference tree (mindspore-ai/acctransformer):
+ *   T = train/acctransformer/flash_attention/ops/flash_attention
+ *   L = train/acctransformer/flash_attention/nn/layer
+ *
+ * Operator semantics (identical to the reference kernels, T/flash_attention_fwd.py
+ * and T/flash_attention_bwd.py; blocks are 128 rows / 128 columns):
+ *
+ *   band(i,j) := j/128 - next_block_num <= i/128 <= j/128 + prev_block_num
+ *   S[i,j] = scale * sum_d q[i,d] k[j,d] + alibi[b,h,(i|0),j] - 10000 * mask[(b|0),i,j]   for band(i,j)
+ *   m = rowmax S;  Pt = exp(S - m);  l = rowsum Pt   (l is taken BEFORE dropout)
+ *   LSE = m + ln l
+ *   O = (Pt / l) * (drop / keep_prob) * v
+ *   backward:  P = exp(S - LSE); Pd = P*drop/keep_prob; dV = Pd^T dO; dP = (dO v^T)*drop/keep_prob
+ *              Dl = rowsum(dO*O); dS = P*(dP - Dl); dQ = scale dS k; dK = scale dS^T q
+ */
+#ifndef ACCT_FA_H_
+#define ACCT_FA_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ACCT_FA_VERSION 100
+
+/* error codes (0 = success) */
+#define ACCT_OK          0
+#define ACCT_E_NULLPTR  (-1)   /* a required pointer is NULL */
+#define ACCT_E_SHAPE    (-2)   /* non-positive or inconsistent extent / stride */
+#define ACCT_E_DTYPE    (-3)   /* dtype is neither ACCT_F16 nor ACCT_BF16 */
+#define ACCT_E_HEADDIM  (-4)   /* D unsupported (supported: 64, 80, 128) */
+#define ACCT_E_ARCH     (-5)   /* current device is not gfx950 */
+#define ACCT_E_LAUNCH   (-6)   /* HIP reported a launch error */
+#define ACCT_E_WORKSPACE (-7)  /* workspace missing or too small */
+#define ACCT_E_PARAM    (-8)   /* scale <= 0, keep_prob outside (0,1], bad mask_kind ... */
+
+#define ACCT_F16  0
+#define ACCT_BF16 1
+
+/* attn_mask interpretation */
+#define ACCT_MASK_NONE     0
+#define ACCT_MASK_DENSE_U8 1   /* uint8 [1|B, Sq, Sk], nonzero = masked (adds -10000); T/attention.py:357-371 */
+#define ACCT_MASK_TILE_U8  3   /* uint8 [128,128] tile applied only where q_blk == kv_blk:
+                                  the reference's compact causal mode, T/attention.py:279-285,363-365 */
+#define ACCT_MASK_CAUSAL   4   /* no tensor: -10000 added where j > i, evaluated by index compare */
+
+#define ACCT_BLOCK_UNBOUNDED 65536   /* default prev/next_block_num, L/flash_attention.py:95-96 */
+
+/*
+ * One description of the problem for forward and backward.  Replaces the
+ * tensor-descriptor dicts handed to the reference's kernel builders
+ * (T/flash_attention_fwd.py:498-530, T/flash_attention_bwd.py:436-477) and
+ * the primitive attrs prev_block_num / next_block_num
+ * (T/flash_attention_impl.py:146-148).
+ */
+typedef struct acct_fa_params {
+  int32_t dtype;                 /* ACCT_F16 | ACCT_BF16: type of q,k,v,O,dO,dQ,dK,dV and alibi */
+  int32_t B, N, Sq, Sk, D;       /* q [B,N,Sq,D]; k,v [B,N,Sk,D] */
+  float   scale;                 /* multiplies q k^T in fp32; 1.0 = the raw reference op, the
+                                    layer passes fp16(D^-1/4)^2 (L/flash_attention.py:117,188-189) */
+  float   keep_prob;             /* 1.0 = no dropout; P *= drop / keep_prob (T/attention.py:373-395) */
+  int32_t prev_block_num;        /* band, in 128-row blocks (T/attention.py:162-167) */
+  int32_t next_block_num;        /* 0 = causal block skip */
+  int32_t mask_kind;             /* ACCT_MASK_* */
+  int32_t reserved0;
+  int64_t mask_stride_b;         /* elements between batches of attn_mask; 0 = broadcast [1,Sq,Sk] */
+  int64_t alibi_stride_b;        /* alibi element strides; stride_q = 0 is the reference's   */
+  int64_t alibi_stride_h;        /* [B,N,1,Sk] row-bias form (L/flash_attention.py:185);      */
+  int64_t alibi_stride_q;        /* stride_b = 0 / stride_h = 0 broadcast over batch / heads  */
+  /* element strides (batch, head, row) of q/dQ, k/dK, v/dV and O/dO; the last
+     dimension is contiguous.  All zeros = contiguous BNSD. */
+  int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3];
+  const void*    q;
+  const void*    k;
+  const void*    v;
+  const uint8_t* attn_mask;      /* per mask_kind; NULL when NONE / CAUSAL */
+  const uint8_t* drop_mask;      /* uint8 [B,N,Sq,Sk] of {0,1}, contiguous; NULL = no dropout */
+  const void*    alibi;          /* dtype, see strides; NULL = none (T/attention.py:347-355) */
+} acct_fa_params;
+
+/* Forward: replaces the `flash_attention` TBE custom op, T/flash_attention_fwd.py:498-530
+ * (outputs `output` and `rowsum`, T/flash_attention_impl.py:129-154).
+ * O is [B,N,Sq,D] in p->dtype with p->o_stride; LSE is fp32 [B,N,Sq] contiguous
+ * (L = m + ln l, T/flash_attention_fwd.py:302-306).  `workspace` must hold
+ * acct_fa_fwd_workspace_bytes(p) bytes (0 unless mask_kind == DENSE_U8). */
+int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE,
+                void* workspace, size_t workspace_bytes, void* stream);
+size_t acct_fa_fwd_workspace_bytes(const acct_fa_params* p);
+
+/* Backward: replaces the `flash_attention_grad` TBE custom op,
+ * T/flash_attention_bwd.py:436-477 (the bprop of T/flash_attention_impl.py:117-124
+ * casts its fp32 results to fp16; here dQ,dK,dV are written in p->dtype directly,
+ * accumulated in fp32 registers).  O and dO use p->o_stride; dQ,dK,dV use the
+ * strides of q,k,v.  Deterministic: no atomics. */
+int acct_fa_bwd(const acct_fa_params* p, const void* O, const void* dO, const float* LSE,
+                void* dQ, void* dK, void* dV,
+                void* workspace, size_t workspace_bytes, void* stream);
+size_t acct_fa_bwd_workspace_bytes(const acct_fa_params* p);
+
+/* Thread-local text of the last error on the calling thread ("" if none).
+ * Stands in for the Python exceptions the reference raises at build time
+ * (L/flash_attention.py:105-108,193-196). */
+const char* acct_last_error(void);
+
+/* ACCT_FA_VERSION of the loaded library. */
+int acct_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* ACCT_FA_H_ */
