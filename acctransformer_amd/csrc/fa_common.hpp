@@ -130,4 +130,41 @@ ACCT_DEV void load_bias4(const T* row, int kv, int limit, bool vec_ok, float out
   }
 }
 
+// ---- 64-row tiles staged through LDS ---------------------------------------
+template <int D> struct TileCfg {
+  static constexpr int KS = D / 16;             // 16-wide k-steps across the head dim
+  static constexpr int DB = (D + 31) / 32;      // 32-wide blocks across the head dim
+  static constexpr int DP = DB * 32;
+  static constexpr int CPR = D / 8;             // 16-byte chunks per row
+  static constexpr int ROWB = DP * 2 + 16;      // LDS row pitch (bytes): +16 keeps b128 reads conflict free
+  static constexpr int BN = 64;                 // rows per staged tile
+  static constexpr int TILEB = BN * ROWB;
+  static constexpr int NLD = (BN * CPR + 255) / 256;
+};
+
+template <typename T, int D>
+ACCT_DEV void tile_load(const T* base, int64_t row_stride, int row0, int nrows, u32x4 (&reg)[TileCfg<D>::NLD]) {
+  using C = TileCfg<D>;
+#pragma unroll
+  for (int i = 0; i < C::NLD; i++) {
+    const int idx = threadIdx.x + 256 * i;
+    const int row = idx / C::CPR, ch = idx % C::CPR;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (idx < C::BN * C::CPR && row0 + row < nrows)
+      v = *reinterpret_cast<const u32x4*>(base + (int64_t)(row0 + row) * row_stride + ch * 8);
+    reg[i] = v;
+  }
+}
+
+template <int D>
+ACCT_DEV void tile_store(ACCT_LDS char* buf, const u32x4 (&reg)[TileCfg<D>::NLD]) {
+  using C = TileCfg<D>;
+#pragma unroll
+  for (int i = 0; i < C::NLD; i++) {
+    const int idx = threadIdx.x + 256 * i;
+    const int row = idx / C::CPR, ch = idx % C::CPR;
+    if (idx < C::BN * C::CPR) *reinterpret_cast<ACCT_LDS u32x4*>(buf + row * C::ROWB + ch * 16) = reg[i];
+  }
+}
+
 }  // namespace acct

@@ -18,47 +18,11 @@
 
 namespace acct {
 
-template <int D> struct FwdCfg {
-  static constexpr int KS = D / 16;             // k-steps of K Q^T
-  static constexpr int DB = (D + 31) / 32;      // 32-row blocks of O^T
-  static constexpr int DP = DB * 32;
-  static constexpr int CPR = D / 8;             // 16-byte chunks per row
-  static constexpr int ROWB = DP * 2 + 16;      // LDS row pitch (bytes): +16 keeps b128 reads conflict free
-  static constexpr int BN = 64;                 // kv rows per tile
-  static constexpr int TILEB = BN * ROWB;
-  static constexpr int NLD = (BN * CPR + 255) / 256;
-};
-
-template <typename T, int D>
-ACCT_DEV void tile_load(const T* base, int64_t row_stride, int row0, int nrows, u32x4 (&reg)[FwdCfg<D>::NLD]) {
-  using C = FwdCfg<D>;
-#pragma unroll
-  for (int i = 0; i < C::NLD; i++) {
-    const int idx = threadIdx.x + 256 * i;
-    const int row = idx / C::CPR, ch = idx % C::CPR;
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (idx < C::BN * C::CPR && row0 + row < nrows)
-      v = *reinterpret_cast<const u32x4*>(base + (int64_t)(row0 + row) * row_stride + ch * 8);
-    reg[i] = v;
-  }
-}
-
-template <int D>
-ACCT_DEV void tile_store(ACCT_LDS char* buf, const u32x4 (&reg)[FwdCfg<D>::NLD]) {
-  using C = FwdCfg<D>;
-#pragma unroll
-  for (int i = 0; i < C::NLD; i++) {
-    const int idx = threadIdx.x + 256 * i;
-    const int row = idx / C::CPR, ch = idx % C::CPR;
-    if (idx < C::BN * C::CPR) *reinterpret_cast<ACCT_LDS u32x4*>(buf + row * C::ROWB + ch * 16) = reg[i];
-  }
-}
-
 template <typename T, int D, int QG, bool GENERAL>
 __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
   using E = Elem<T>;
   using V8 = typename E::V8;
-  using C = FwdCfg<D>;
+  using C = TileCfg<D>;
   constexpr int BM = 128 * QG;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 buffers][K tile | V tile]
@@ -313,7 +277,7 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
 
 template <typename T, int D, int QG, bool GENERAL>
 static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
-  using C = FwdCfg<D>;
+  using C = TileCfg<D>;
   constexpr int BM = 128 * QG;
   a.n_tiles = (a.Sq + BM - 1) / BM;
   const size_t smem = 4 * (size_t)C::TILEB;
