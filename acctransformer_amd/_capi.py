@@ -32,7 +32,7 @@ class AcctFaParams(ctypes.Structure):
         ("D", ctypes.c_int32),
         ("scale", ctypes.c_float), ("keep_prob", ctypes.c_float),
         ("prev_block_num", ctypes.c_int32), ("next_block_num", ctypes.c_int32),
-        ("mask_kind", ctypes.c_int32), ("reserved0", ctypes.c_int32),
+        ("mask_kind", ctypes.c_int32), ("row_block_prefix", ctypes.c_int32),
         ("mask_stride_b", ctypes.c_int64),
         ("alibi_stride_b", ctypes.c_int64), ("alibi_stride_h", ctypes.c_int64), ("alibi_stride_q", ctypes.c_int64),
         ("q_stride", ctypes.c_int64 * 3), ("k_stride", ctypes.c_int64 * 3),
@@ -99,7 +99,7 @@ def _bhs_strides(t):
 
 
 def make_params(q, k, v, *, scale, keep_prob=1.0, prev_block_num=BLOCK_UNBOUNDED, next_block_num=BLOCK_UNBOUNDED,
-                mask_kind=MASK_NONE, attn_mask=None, drop_mask=None, alibi=None, o_like=None):
+                mask_kind=MASK_NONE, attn_mask=None, drop_mask=None, alibi=None, o_like=None, row_block_prefix=0):
     """Describe one attention problem.  q [B,N,Sq,D]; k,v [B,N,Sk,D] (any
     batch/head/row strides, unit stride along D); attn_mask uint8 [1|B,Sq,Sk]
     (DENSE) or [128,128] (TILE); drop_mask uint8 [B,N,Sq,Sk]; alibi in q's
@@ -124,6 +124,7 @@ def make_params(q, k, v, *, scale, keep_prob=1.0, prev_block_num=BLOCK_UNBOUNDED
     p.scale, p.keep_prob = float(scale), float(keep_prob)
     p.prev_block_num, p.next_block_num = int(min(prev_block_num, BLOCK_UNBOUNDED)), int(min(next_block_num, BLOCK_UNBOUNDED))
     p.mask_kind = mask_kind
+    p.row_block_prefix = int(row_block_prefix)
     p.q_stride, p.k_stride, p.v_stride = _bhs_strides(q), _bhs_strides(k), _bhs_strides(v)
     if o_like is not None:
         p.o_stride = _bhs_strides(o_like)

@@ -60,6 +60,7 @@ int validate(const acct_fa_params* p) {
   if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return fail(ACCT_E_PARAM, "scale must be positive and finite, got %g", (double)p->scale);
   if (!(p->keep_prob > 0.f && p->keep_prob <= 1.f)) return fail(ACCT_E_PARAM, "keep_prob must be in (0, 1], got %g", (double)p->keep_prob);
   if (p->prev_block_num < 0 || p->next_block_num < 0) return fail(ACCT_E_PARAM, "prev_block_num / next_block_num must be >= 0");
+  if (p->row_block_prefix < 0 || p->row_block_prefix % 128 != 0) return fail(ACCT_E_PARAM, "row_block_prefix must be 0 or a positive multiple of 128, got %d", p->row_block_prefix);
   switch (p->mask_kind) {
     case ACCT_MASK_NONE: case ACCT_MASK_CAUSAL: break;
     case ACCT_MASK_DENSE_U8: case ACCT_MASK_TILE_U8:
@@ -112,11 +113,8 @@ acct::FaArgs make_args(const acct_fa_params* p) {
   a.prev_blk = p->prev_block_num > ACCT_BLOCK_UNBOUNDED ? ACCT_BLOCK_UNBOUNDED : p->prev_block_num;
   a.next_blk = p->next_block_num > ACCT_BLOCK_UNBOUNDED ? ACCT_BLOCK_UNBOUNDED : p->next_block_num;
   a.mask_kind = p->mask_kind;
+  a.row_prefix = p->row_block_prefix;
   return a;
-}
-
-bool is_general(const acct_fa_params* p) {
-  return p->mask_kind == ACCT_MASK_DENSE_U8 || p->mask_kind == ACCT_MASK_TILE_U8 || p->drop_mask || p->alibi;
 }
 
 size_t flag_bytes(const acct_fa_params* p) {
@@ -171,7 +169,7 @@ int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, s
   // 64 query rows per wave (256 per workgroup) once that still fills the chip
   int qg = ((long long)p->B * p->N * ((p->Sq + 255) / 256) >= n_cu) ? 2 : 1;
   qg = env_int("ACCT_FA_FWD_QG", qg) == 1 ? 1 : 2;
-  hipError_t e = acct::launch_fwd(a, p->dtype, p->D, is_general(p), qg, st);
+  hipError_t e = acct::launch_fwd(a, p->dtype, p->D, qg, st);
   if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "forward kernel: %s", hipGetErrorString(e));
   return ACCT_OK;
 }
@@ -203,7 +201,7 @@ int acct_fa_bwd(const acct_fa_params* p, const void* O, const void* dO, const fl
     hipError_t e = acct::launch_mask_blocks(a, flags, p->mask_stride_b ? p->B : 1, st);
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
   }
-  hipError_t e = acct::launch_bwd(a, p->dtype, p->D, is_general(p), st);
+  hipError_t e = acct::launch_bwd(a, p->dtype, p->D, st);
   if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "backward kernels: %s", hipGetErrorString(e));
   return ACCT_OK;
 }

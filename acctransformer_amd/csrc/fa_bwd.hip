@@ -42,7 +42,7 @@ ACCT_DEV typename Elem<T>::V8 pack8(const float* x) {
 // ============================================================================
 // dQ kernel (and delta): query-tile owner, structure of the forward kernel
 // ============================================================================
-template <typename T, int D, int QG, bool GENERAL>
+template <typename T, int D, int QG, bool BIAS, bool DROP>
 __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
   using E = Elem<T>;
   using V8 = typename E::V8;
@@ -72,7 +72,9 @@ __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
   int j_lo = kvb_lo * 2, j_hi = min(kvb_hi * 2 + 1, (a.Sk - 1) / 64);
   const bool causal = a.mask_kind == kMaskCausal;
   if (causal) j_hi = min(j_hi, (q_end - 1) / 64);
+  if (a.row_prefix) j_hi = min(j_hi, (((q_end - 1) / a.row_prefix + 1) * a.row_prefix - 1) / 64);
   const int wqb = wq0 / 128;
+  const int wkv_limit = a.row_prefix ? (wq0 / a.row_prefix + 1) * a.row_prefix : 0x7fffffff;
 
   // Q and dO fragments (B operands), delta and L of the lane's query row
   V8 qf[QG][C::KS], dof[QG][C::KS];
@@ -112,13 +114,13 @@ __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
       for (int r = 0; r < 16; r++) acc[gq][db][r] = 0.f;
 
   const int mb = a.mask_sb ? b : 0;
-  const uint8_t* maskp = GENERAL && a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
-  const uint8_t* dropp = GENERAL && a.drop ? a.drop + ((int64_t)bh * a.Sq) * a.Sk : nullptr;
-  const T* alibip = GENERAL && a.alibi ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
-  const bool mask_vec = GENERAL && (a.mask_kind == kMaskDense ? (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0
-                                                              : ((uintptr_t)a.mask & 3) == 0);
-  const bool drop_vec = GENERAL && (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 3) == 0;
-  const bool alibi_vec = GENERAL && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
+  const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
+  const uint8_t* dropp = DROP ? a.drop + ((int64_t)bh * a.Sq) * a.Sk : nullptr;
+  const T* alibip = BIAS ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
+  const bool mask_vec = a.mask_kind == kMaskDense ? (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0
+                                                  : ((uintptr_t)a.mask & 3) == 0;
+  const bool drop_vec = DROP && (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 3) == 0;
+  const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
   if (j_lo <= j_hi) {
     u32x4 kreg[C::NLD], vreg[C::NLD];
@@ -141,16 +143,17 @@ __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
       const int kvb = j >> 1;
       bool act = (kvb - a.next_blk <= wqb) && (wqb <= kvb + a.prev_blk) && (wq0 < a.Sq);
       if (causal) act = act && (kv0 <= wq_end - 1);
+      act = act && (kv0 < wkv_limit);
       bool apply_mask = false;
-      if (GENERAL) {
-        if (a.mask_kind == kMaskDense && act) {
-          const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + wqb) * a.Tc + kvb];
-          act = f != kBlkSkip;
-          apply_mask = f == kBlkApply;
-        } else if (a.mask_kind == kMaskTile) {
-          apply_mask = wqb == kvb;
-        }
+      if (a.mask_kind == kMaskDense && act) {
+        const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + wqb) * a.Tc + kvb];
+        act = f != kBlkSkip;
+        apply_mask = f == kBlkApply;
+      } else if (a.mask_kind == kMaskTile) {
+        apply_mask = wqb == kvb;
       }
+      const bool diag = causal && (kv0 + 63 > wq0);
+      const bool tail = kv0 + 64 > a.Sk;
       if (act) {
         V8 dsf[QG][2][2];
 #pragma unroll
@@ -181,27 +184,24 @@ __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
               const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
               float bias[4] = {0.f, 0.f, 0.f, 0.f};
               uint32_t mbits = 0, dbits = 0x01010101u;
-              if (GENERAL) {
-                if (alibip) load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
-                if (apply_mask) {
-                  if (a.mask_kind == kMaskDense) mbits = load_u8x4(maskp + (int64_t)qrow_c * a.Sk, kv, a.Sk, mask_vec);
-                  else mbits = load_u8x4(maskp + (qrow_c & 127) * 128, kv & 127, 128, mask_vec);
-                }
-                if (dropp) dbits = load_u8x4(dropp + (int64_t)qrow_c * a.Sk, kv, a.Sk, drop_vec);
+              if (BIAS) load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
+              if (apply_mask) {
+                if (a.mask_kind == kMaskDense) mbits = load_u8x4(maskp + (int64_t)qrow_c * a.Sk, kv, a.Sk, mask_vec);
+                else mbits = load_u8x4(maskp + (qrow_c & 127) * 128, kv & 127, 128, mask_vec);
               }
+              if (DROP) dbits = load_u8x4(dropp + (int64_t)qrow_c * a.Sk, kv, a.Sk, drop_vec);
 #pragma unroll
               for (int e = 0; e < 4; e++) {
                 const int r = 4 * r4 + e;
-                float x = s[gq][r] * a.scale_log2e;
-                if (GENERAL) {
-                  x += bias[e] * kLog2e;
-                  if ((mbits >> (8 * e)) & 0xffu) x += kMaskFill * kLog2e;
+                float x = __builtin_fmaf(s[gq][r], a.scale_log2e, -lq[gq]);
+                if (BIAS) x = __builtin_fmaf(bias[e], kLog2e, x);
+                if (apply_mask || diag) {
+                  if (((mbits >> (8 * e)) & 0xffu) || (causal && kv + e > qrow)) x += kMaskFill * kLog2e;
                 }
-                if (causal && kv + e > qrow) x += kMaskFill * kLog2e;
-                float p = fast_exp2(x - lq[gq]);
-                if (kv + e >= a.Sk) p = 0.f;
+                float p = fast_exp2(x);
+                if (tail && kv + e >= a.Sk) p = 0.f;
                 float dpv = dp[gq][r];
-                if (GENERAL && dropp) dpv = ((dbits >> (8 * e)) & 0xffu) ? dpv * a.inv_keep : 0.f;
+                if (DROP) dpv = ((dbits >> (8 * e)) & 0xffu) ? dpv * a.inv_keep : 0.f;
                 ds[r] = p * (dpv - dl[gq]);
               }
             }
@@ -258,7 +258,7 @@ __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
 // dK/dV kernel: kv-tile owner.  Each wave owns 32*KG key rows; Q and dO tiles of
 // 64 query rows are staged through LDS.
 // ============================================================================
-template <typename T, int D, int KG, bool GENERAL>
+template <typename T, int D, int KG, bool BIAS, bool DROP>
 __global__ void __launch_bounds__(256) fa_bwd_dkdv_kernel(const FaArgs a) {
   using E = Elem<T>;
   using V8 = typename E::V8;
@@ -316,9 +316,9 @@ __global__ void __launch_bounds__(256) fa_bwd_dkdv_kernel(const FaArgs a) {
       for (int r = 0; r < 16; r++) { dk[gk][db][r] = 0.f; dv[gk][db][r] = 0.f; }
 
   const int mb = a.mask_sb ? b : 0;
-  const uint8_t* maskp = GENERAL && a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
-  const uint8_t* dropp = GENERAL && a.drop ? a.drop + ((int64_t)bh * a.Sq) * a.Sk : nullptr;
-  const T* alibip = GENERAL && a.alibi ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
+  const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
+  const uint8_t* dropp = DROP ? a.drop + ((int64_t)bh * a.Sq) * a.Sk : nullptr;
+  const T* alibip = BIAS ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
   const bool stat_vec = ((((uintptr_t)lsep | (uintptr_t)delp) & 15) == 0);
 
   if (i_lo <= i_hi) {
@@ -342,16 +342,16 @@ __global__ void __launch_bounds__(256) fa_bwd_dkdv_kernel(const FaArgs a) {
       const int qb = i >> 1;
       bool act = (wkb - a.next_blk <= qb) && (qb <= wkb + a.prev_blk) && (wk0 < a.Sk);
       if (causal) act = act && (qt0 + 63 >= wk0);
+      if (a.row_prefix) act = act && (wk0 < (qt0 / a.row_prefix + 1) * a.row_prefix);
       bool apply_mask = false;
-      if (GENERAL) {
-        if (a.mask_kind == kMaskDense && act) {
-          const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + qb) * a.Tc + wkb];
-          act = f != kBlkSkip;
-          apply_mask = f == kBlkApply;
-        } else if (a.mask_kind == kMaskTile) {
-          apply_mask = wkb == qb;
-        }
+      if (a.mask_kind == kMaskDense && act) {
+        const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + qb) * a.Tc + wkb];
+        act = f != kBlkSkip;
+        apply_mask = f == kBlkApply;
+      } else if (a.mask_kind == kMaskTile) {
+        apply_mask = wkb == qb;
       }
+      const bool diag = causal && (wk0 + 32 * KG - 1 > qt0);
       if (act) {
 #pragma unroll
         for (int c = 0; c < 2; c++) {                 // 32-row query chunk of the tile
@@ -388,23 +388,21 @@ __global__ void __launch_bounds__(256) fa_bwd_dkdv_kernel(const FaArgs a) {
             for (int r = 0; r < 16; r++) {
               const int q = qt0 + 32 * c + 8 * (r >> 2) + 4 * g + (r & 3);
               const int q_c = min(q, a.Sq - 1);
-              float x = s[gk][r] * a.scale_log2e;
+              float x = __builtin_fmaf(s[gk][r], a.scale_log2e, -lrow[r] * kLog2e);
               bool keep = true;
-              if (GENERAL) {
-                if (alibip) x += (float)alibip[(int64_t)q_c * a.al_sq + kv_c] * kLog2e;
-                if (apply_mask) {
-                  const uint8_t mbyte = a.mask_kind == kMaskDense ? maskp[(int64_t)q_c * a.Sk + kv_c]
-                                                                  : maskp[(q_c & 127) * 128 + (kv_c & 127)];
-                  if (mbyte) x += kMaskFill * kLog2e;
-                }
-                if (dropp) keep = dropp[(int64_t)q_c * a.Sk + kv_c] != 0;
+              if (BIAS) x = __builtin_fmaf((float)alibip[(int64_t)q_c * a.al_sq + kv_c], kLog2e, x);
+              if (apply_mask) {
+                const uint8_t mbyte = a.mask_kind == kMaskDense ? maskp[(int64_t)q_c * a.Sk + kv_c]
+                                                                : maskp[(q_c & 127) * 128 + (kv_c & 127)];
+                if (mbyte) x += kMaskFill * kLog2e;
               }
-              if (causal && kv > q) x += kMaskFill * kLog2e;
-              float p = fast_exp2(x - lrow[r] * kLog2e);
+              if (DROP) keep = dropp[(int64_t)q_c * a.Sk + kv_c] != 0;
+              if (diag && kv > q) x += kMaskFill * kLog2e;
+              float p = fast_exp2(x);
               if (kv >= a.Sk) p = 0.f;
               float dpv = dp[gk][r];
               float pd = p;
-              if (GENERAL && dropp) {
+              if (DROP) {
                 dpv = keep ? dpv * a.inv_keep : 0.f;
                 pd = keep ? p * a.inv_keep : 0.f;
               }
@@ -470,7 +468,7 @@ __global__ void __launch_bounds__(256) fa_bwd_dkdv_kernel(const FaArgs a) {
 }
 
 // ---- launchers ----------------------------------------------------------------
-template <typename T, int D, bool GENERAL>
+template <typename T, int D, bool BIAS, bool DROP>
 static hipError_t launch_bwd_t(FaArgs a, hipStream_t st) {
   using C = TileCfg<D>;
   const size_t smem = 4 * (size_t)C::TILEB;
@@ -478,7 +476,7 @@ static hipError_t launch_bwd_t(FaArgs a, hipStream_t st) {
   {
     constexpr int QG = 1;
     a.n_tiles = (a.Sq + 128 * QG - 1) / (128 * QG);
-    auto kern = fa_bwd_dq_kernel<T, D, QG, GENERAL>;
+    auto kern = fa_bwd_dq_kernel<T, D, QG, BIAS, DROP>;
     e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)((long long)a.n_tiles * a.B * a.N)), dim3(256), smem, st, a);
@@ -488,7 +486,7 @@ static hipError_t launch_bwd_t(FaArgs a, hipStream_t st) {
   {
     constexpr int KG = 1;
     a.n_tiles = (a.Sk + 128 * KG - 1) / (128 * KG);
-    auto kern = fa_bwd_dkdv_kernel<T, D, KG, GENERAL>;
+    auto kern = fa_bwd_dkdv_kernel<T, D, KG, BIAS, DROP>;
     e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)((long long)a.n_tiles * a.B * a.N)), dim3(256), smem, st, a);
@@ -498,19 +496,21 @@ static hipError_t launch_bwd_t(FaArgs a, hipStream_t st) {
 }
 
 template <typename T, int D>
-static hipError_t launch_bwd_d(const FaArgs& a, bool general, hipStream_t st) {
-  return general ? launch_bwd_t<T, D, true>(a, st) : launch_bwd_t<T, D, false>(a, st);
+static hipError_t launch_bwd_d(const FaArgs& a, hipStream_t st) {
+  const bool bias = a.alibi != nullptr, drop = a.drop != nullptr;
+  if (bias) return drop ? launch_bwd_t<T, D, true, true>(a, st) : launch_bwd_t<T, D, true, false>(a, st);
+  return drop ? launch_bwd_t<T, D, false, true>(a, st) : launch_bwd_t<T, D, false, false>(a, st);
 }
 
-hipError_t launch_bwd(const FaArgs& a, int dtype, int D, bool general, hipStream_t st) {
+hipError_t launch_bwd(const FaArgs& a, int dtype, int D, hipStream_t st) {
   if (dtype == 0) {
-    if (D == 128) return launch_bwd_d<f16, 128>(a, general, st);
-    if (D == 64) return launch_bwd_d<f16, 64>(a, general, st);
-    if (D == 80) return launch_bwd_d<f16, 80>(a, general, st);
+    if (D == 128) return launch_bwd_d<f16, 128>(a, st);
+    if (D == 64) return launch_bwd_d<f16, 64>(a, st);
+    if (D == 80) return launch_bwd_d<f16, 80>(a, st);
   } else {
-    if (D == 128) return launch_bwd_d<bf16, 128>(a, general, st);
-    if (D == 64) return launch_bwd_d<bf16, 64>(a, general, st);
-    if (D == 80) return launch_bwd_d<bf16, 80>(a, general, st);
+    if (D == 128) return launch_bwd_d<bf16, 128>(a, st);
+    if (D == 64) return launch_bwd_d<bf16, 64>(a, st);
+    if (D == 80) return launch_bwd_d<bf16, 80>(a, st);
   }
   return hipErrorInvalidValue;
 }

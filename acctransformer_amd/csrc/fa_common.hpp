@@ -102,6 +102,7 @@ struct FaArgs {
   float mask_add_raw;                  // -10000 / scale: the mask in raw q.k units
   int prev_blk, next_blk;
   int mask_kind;
+  int row_prefix;                      // >0: row i sees keys j < (i/row_prefix + 1)*row_prefix only (multiple of 128)
   int n_tiles;                         // tiles along the owner dimension
 };
 

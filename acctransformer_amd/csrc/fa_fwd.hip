@@ -18,7 +18,7 @@
 
 namespace acct {
 
-template <typename T, int D, int QG, bool GENERAL>
+template <typename T, int D, int QG, bool BIAS, bool DROP>
 __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
   using E = Elem<T>;
   using V8 = typename E::V8;
@@ -47,7 +47,9 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
   int j_lo = kvb_lo * 2, j_hi = min(kvb_hi * 2 + 1, (a.Sk - 1) / 64);
   const bool causal = a.mask_kind == kMaskCausal;
   if (causal) j_hi = min(j_hi, (q_end - 1) / 64);
+  if (a.row_prefix) j_hi = min(j_hi, (((q_end - 1) / a.row_prefix + 1) * a.row_prefix - 1) / 64);
   const int wqb = wq0 / 128;                                // 128-block of this wave's rows
+  const int wkv_limit = a.row_prefix ? (wq0 / a.row_prefix + 1) * a.row_prefix : 0x7fffffff;   // keys past it are absent
 
   // ---- Q fragments (B operand of K Q^T): lane holds row l32, d = 16t + 8g .. +7 ----
   V8 qf[QG][C::KS];
@@ -73,15 +75,18 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
       for (int r = 0; r < 16; r++) o[gq][db][r] = 0.f;
   }
 
-  const float cmul = GENERAL ? 1.0f : a.scale_log2e;   // exp2 argument = s * cmul - m * cmul
+  // Scores stay in raw q.k units (exp2 argument = s * scale*log2e - m * scale*log2e, one FMA) unless a
+  // bias is added, in which case they are converted to log2 units first.
+  const float cmul = BIAS ? 1.0f : a.scale_log2e;
+  const float madd = BIAS ? kMaskFill * kLog2e : a.mask_add_raw;   // the additive -10000 in the units of s
   const int mb = a.mask_sb ? b : 0;
-  const uint8_t* maskp = GENERAL && a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
-  const uint8_t* dropp = GENERAL && a.drop ? a.drop + ((int64_t)bh * a.Sq) * a.Sk : nullptr;
-  const T* alibip = GENERAL && a.alibi ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
-  const bool mask_vec = GENERAL && (a.mask_kind == kMaskDense ? (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0
-                                                              : ((uintptr_t)a.mask & 3) == 0);
-  const bool drop_vec = GENERAL && (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 3) == 0;
-  const bool alibi_vec = GENERAL && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
+  const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
+  const uint8_t* dropp = DROP ? a.drop + ((int64_t)bh * a.Sq) * a.Sk : nullptr;
+  const T* alibip = BIAS ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
+  const bool mask_vec = a.mask_kind == kMaskDense ? (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0
+                                                  : ((uintptr_t)a.mask & 3) == 0;
+  const bool drop_vec = DROP && (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 3) == 0;
+  const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
   if (j_lo <= j_hi) {
     u32x4 kreg[C::NLD], vreg[C::NLD];
@@ -104,15 +109,14 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
       const int kvb = j >> 1;
       bool act = (kvb - a.next_blk <= wqb) && (wqb <= kvb + a.prev_blk) && (wq0 < a.Sq);
       if (causal) act = act && (kv0 <= wq_end - 1);
+      act = act && (kv0 < wkv_limit);
       bool apply_mask = false;
-      if (GENERAL) {
-        if (a.mask_kind == kMaskDense && act) {
-          const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + wqb) * a.Tc + kvb];
-          act = f != kBlkSkip;
-          apply_mask = f == kBlkApply;
-        } else if (a.mask_kind == kMaskTile) {
-          apply_mask = wqb == kvb;
-        }
+      if (a.mask_kind == kMaskDense && act) {
+        const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + wqb) * a.Tc + kvb];
+        act = f != kBlkSkip;
+        apply_mask = f == kBlkApply;
+      } else if (a.mask_kind == kMaskTile) {
+        apply_mask = wqb == kvb;
       }
       if (act) {
         // ---- S^T = K Q^T : s[gq][c] is the 32(kv) x 32(q) tile of kv chunk c ----
@@ -140,14 +144,25 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
         for (int gq = 0; gq < QG; gq++) {
           const int qrow = wq0 + 32 * gq + l32;
           const int qrow_c = min(qrow, a.Sq - 1);            // clamped for side-input addressing
-          if (GENERAL) {
+          if (BIAS) {
 #pragma unroll
             for (int c = 0; c < 2; c++)
 #pragma unroll
               for (int r4 = 0; r4 < 4; r4++) {
                 const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
-                float bias[4] = {0.f, 0.f, 0.f, 0.f};
-                if (alibip) load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
+                float bias[4];
+                load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                  s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale_log2e, bias[e] * kLog2e);
+              }
+          }
+          if (apply_mask || diag || tail) {
+#pragma unroll
+            for (int c = 0; c < 2; c++)
+#pragma unroll
+              for (int r4 = 0; r4 < 4; r4++) {
+                const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
                 uint32_t mbits = 0;
                 if (apply_mask) {
                   if (a.mask_kind == kMaskDense) mbits = load_u8x4(maskp + (int64_t)qrow_c * a.Sk, kv, a.Sk, mask_vec);
@@ -155,26 +170,12 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
                 }
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                  float x = s[gq][c][4 * r4 + e] * a.scale_log2e + bias[e] * kLog2e;
-                  if ((mbits >> (8 * e)) & 0xffu) x += kMaskFill * kLog2e;
-                  if (causal && kv + e > qrow) x += kMaskFill * kLog2e;
+                  float x = s[gq][c][4 * r4 + e];
+                  if (((mbits >> (8 * e)) & 0xffu) || (causal && kv + e > qrow)) x += madd;
                   if (kv + e >= a.Sk) x = -INFINITY;
                   s[gq][c][4 * r4 + e] = x;
                 }
               }
-          } else {
-            if (diag || tail) {
-#pragma unroll
-              for (int c = 0; c < 2; c++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                  const int kv = kv0 + 32 * c + 8 * (r >> 2) + 4 * g + (r & 3);
-                  float x = s[gq][c][r];
-                  if (causal && kv > qrow) x += a.mask_add_raw;
-                  if (kv >= a.Sk) x = -INFINITY;
-                  s[gq][c][r] = x;
-                }
-            }
           }
           // ---- online softmax for query row qrow ----
           float mx = s[gq][0][0];
@@ -197,7 +198,7 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
               rs += p[c][r];
             }
           lsum[gq] = lsum[gq] * alpha + rs;                  // row sum BEFORE dropout
-          if (GENERAL && dropp) {
+          if (DROP) {
 #pragma unroll
             for (int c = 0; c < 2; c++)
 #pragma unroll
@@ -251,7 +252,7 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
 
   // ---- epilogue: O = O^T / l, LSE = m + ln l ----
   T* op = (T*)a.o + b * a.o_sb + h * a.o_sh;
-  const float mnat = GENERAL ? kLn2 : a.scale;
+  const float mnat = BIAS ? kLn2 : a.scale;
 #pragma unroll
   for (int gq = 0; gq < QG; gq++) {
     const int row = wq0 + 32 * gq + l32;
@@ -275,13 +276,13 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
   }
 }
 
-template <typename T, int D, int QG, bool GENERAL>
+template <typename T, int D, int QG, bool BIAS, bool DROP>
 static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
   using C = TileCfg<D>;
   constexpr int BM = 128 * QG;
   a.n_tiles = (a.Sq + BM - 1) / BM;
   const size_t smem = 4 * (size_t)C::TILEB;
-  auto kern = fa_fwd_kernel<T, D, QG, GENERAL>;
+  auto kern = fa_fwd_kernel<T, D, QG, BIAS, DROP>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (e != hipSuccess) return e;
   const long long nblk = (long long)a.n_tiles * a.B * a.N;
@@ -289,21 +290,27 @@ static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
   return hipGetLastError();
 }
 
-template <typename T, int D>
-static hipError_t launch_fwd_d(const FaArgs& a, bool general, int qg, hipStream_t st) {
-  if (general) return qg == 2 ? launch_fwd_t<T, D, 2, true>(a, st) : launch_fwd_t<T, D, 1, true>(a, st);
-  return qg == 2 ? launch_fwd_t<T, D, 2, false>(a, st) : launch_fwd_t<T, D, 1, false>(a, st);
+template <typename T, int D, int QG>
+static hipError_t launch_fwd_q(const FaArgs& a, hipStream_t st) {
+  const bool bias = a.alibi != nullptr, drop = a.drop != nullptr;
+  if (bias) return drop ? launch_fwd_t<T, D, QG, true, true>(a, st) : launch_fwd_t<T, D, QG, true, false>(a, st);
+  return drop ? launch_fwd_t<T, D, QG, false, true>(a, st) : launch_fwd_t<T, D, QG, false, false>(a, st);
 }
 
-hipError_t launch_fwd(const FaArgs& a, int dtype, int D, bool general, int qg, hipStream_t st) {
+template <typename T, int D>
+static hipError_t launch_fwd_d(const FaArgs& a, int qg, hipStream_t st) {
+  return qg == 2 ? launch_fwd_q<T, D, 2>(a, st) : launch_fwd_q<T, D, 1>(a, st);
+}
+
+hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st) {
   if (dtype == 0) {
-    if (D == 128) return launch_fwd_d<f16, 128>(a, general, qg, st);
-    if (D == 64) return launch_fwd_d<f16, 64>(a, general, qg, st);
-    if (D == 80) return launch_fwd_d<f16, 80>(a, general, qg, st);
+    if (D == 128) return launch_fwd_d<f16, 128>(a, qg, st);
+    if (D == 64) return launch_fwd_d<f16, 64>(a, qg, st);
+    if (D == 80) return launch_fwd_d<f16, 80>(a, qg, st);
   } else {
-    if (D == 128) return launch_fwd_d<bf16, 128>(a, general, qg, st);
-    if (D == 64) return launch_fwd_d<bf16, 64>(a, general, qg, st);
-    if (D == 80) return launch_fwd_d<bf16, 80>(a, general, qg, st);
+    if (D == 128) return launch_fwd_d<bf16, 128>(a, qg, st);
+    if (D == 64) return launch_fwd_d<bf16, 64>(a, qg, st);
+    if (D == 80) return launch_fwd_d<bf16, 80>(a, qg, st);
   }
   return hipErrorInvalidValue;
 }

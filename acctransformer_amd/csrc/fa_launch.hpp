@@ -4,12 +4,12 @@
 
 namespace acct {
 
-// forward: qg = query groups of 32 rows per wave (1 or 2); general = side inputs
-// (dense/tile mask, dropout mask, alibi) present
-hipError_t launch_fwd(const FaArgs& a, int dtype, int D, bool general, int qg, hipStream_t st);
+// forward: qg = query groups of 32 rows per wave (1 or 2); the bias / dropout
+// variants are picked from a.alibi / a.drop
+hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st);
 
 // backward: delta pre-pass, dK/dV kernel (kv-tile owner) and dQ kernel (q-tile owner)
-hipError_t launch_bwd(const FaArgs& a, int dtype, int D, bool general, hipStream_t st);
+hipError_t launch_bwd(const FaArgs& a, int dtype, int D, hipStream_t st);
 
 // classify the 128x128 blocks of a dense uint8 mask into clean / apply / skip
 hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, int MB, hipStream_t st);

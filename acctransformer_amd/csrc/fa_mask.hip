@@ -21,7 +21,8 @@ __global__ void __launch_bounds__(256) fa_mask_blocks_kernel(const FaArgs a, uin
   const uint8_t* mrow = a.mask + (int64_t)mb * a.mask_sb + (int64_t)min(row, a.Sq - 1) * a.Sk;
   const bool vec_ok = (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0;
   uint8_t* frow = flags + ((int64_t)mb * a.Tr + qb) * a.Tc;
-  const int lo = max(0, qb - a.prev_blk), hi = min(a.Tc - 1, qb + a.next_blk);
+  int lo = max(0, qb - a.prev_blk), hi = min(a.Tc - 1, qb + a.next_blk);
+  if (a.row_prefix) hi = min(hi, ((qb * 128 / a.row_prefix + 1) * a.row_prefix - 1) / 128);
   for (int kvb = tid; kvb < a.Tc; kvb += 256)
     if (kvb < lo || kvb > hi) frow[kvb] = kBlkClean;
   bool row_unmasked = false;

@@ -1,0 +1,187 @@
+"""Operator binding of the FlashAttention2 forward / backward kernels.
+
+Mirrors train/acctransformer/flash_attention/ops/flash_attention/flash_attention_impl.py:96-154
+of the reference: `get_flash_attention(prev_block_num, next_block_num,
+tiling_stgy_name)` returns the forward primitive
+`(query, key, value, attn_mask, dropout_mask, alibi_mask) -> (output, rowsum)`
+with its gradient attached, and `get_flash_attention_grad(...)` returns
+`bprop(query, key, value, attn_mask, dropout_mask, alibi_mask, outs, douts)
+-> (dq, dk, dv, 0, 0, 0)`.  Where the reference hands tensor descriptors to a
+TBE kernel builder, this module hands device pointers to the C ABI of
+libacct_fa.so; torch supplies memory, streams and autograd plumbing only.
+
+Differences from the reference that a caller can see:
+  * `scale` (default 1.0, the raw op) is applied to q k^T inside the kernel in
+    fp32; the reference's layer pre-multiplies q and k instead.
+  * masks may be uint8/bool as well as floating; a floating attn_mask is read
+    as "nonzero = masked" (the reference multiplies its value by -10000, and
+    only ever feeds 0/1).  A floating dropout_mask is the reference's
+    {0, 1/keep_prob} form; a uint8/bool one is {0,1} with `keep_prob` given.
+  * dq, dk, dv come back in q's dtype directly (the reference returns fp32
+    and casts to fp16 in bprop, flash_attention_impl.py:121-123).
+"""
+from __future__ import annotations
+
+import weakref
+
+import torch
+
+from acctransformer_amd import _capi
+
+TILING_BLOCK_SIZE = 128                       # constants.py:19 of the reference ops
+_STRATEGIES = ("sparse", "wukong")            # tiling_strategy/sparse_tiling.py, wukong_tiling.py
+
+
+def _check_strategy(name):
+    # tiling_strategy/strategy.py:51-58: unknown names raise at construction
+    if name not in _STRATEGIES:
+        raise Exception(f"Strategy:{name} not supported")
+
+
+# ---- attn_mask classification ------------------------------------------------
+_mask_cache = {}
+
+
+def _is_compact_shape(shape):
+    """attention.py:279-285 (is_only_causal_mask): (128,128) or (1,128,128)."""
+    if len(shape) == 2:
+        return shape[0] == TILING_BLOCK_SIZE and shape[1] == TILING_BLOCK_SIZE
+    if len(shape) == 3:
+        return shape[0] == 1 and shape[1] == TILING_BLOCK_SIZE and shape[2] == TILING_BLOCK_SIZE
+    return False
+
+
+def _classify_mask(attn_mask, Sq, Sk):
+    """Returns (mask_kind, uint8 tensor or None).  The outcome is remembered per
+    tensor object and version, so a mask reused across steps is inspected once."""
+    key = id(attn_mask)
+    hit = _mask_cache.get(key)
+    if hit is not None and hit[0]() is attn_mask and hit[1] == attn_mask._version and hit[2] == (Sq, Sk):
+        return hit[3], hit[4]
+    if attn_mask.dtype in (torch.uint8, torch.bool):
+        m8 = attn_mask.contiguous().view(torch.uint8) if attn_mask.dtype == torch.bool else attn_mask.contiguous()
+    else:
+        m8 = attn_mask.ne(0).to(torch.uint8)
+    compact = _is_compact_shape(tuple(attn_mask.shape)) and not (Sq == TILING_BLOCK_SIZE and Sk == TILING_BLOCK_SIZE
+                                                                  and attn_mask.dim() == 3)
+    if compact:
+        tri = torch.triu(torch.ones(128, 128, dtype=torch.uint8, device=m8.device), diagonal=1)
+        if torch.equal(m8.reshape(128, 128), tri):
+            kind, out = _capi.MASK_CAUSAL, None      # evaluated by index compare, no loads
+        else:
+            kind, out = _capi.MASK_TILE_U8, m8.reshape(128, 128)
+        compact_kind = True
+    else:
+        compact_kind = False
+        if m8.dim() == 2:
+            m8 = m8.unsqueeze(0)
+        if m8.dim() != 3 or m8.shape[1] != Sq or m8.shape[2] != Sk:
+            raise ValueError(f"attn_mask must be [1|B,{Sq},{Sk}] or a (1,128,128) causal tile, got {tuple(attn_mask.shape)}")
+        kind, out = _capi.MASK_DENSE_U8, m8
+        if Sq == Sk:
+            rows = torch.arange(Sq, device=m8.device)
+            tri = (rows[None, :] > rows[:, None]).to(torch.uint8)
+            if all(torch.equal(m8[i], tri) for i in range(m8.shape[0])):
+                kind, out = _capi.MASK_CAUSAL, None
+    if len(_mask_cache) > 64:
+        for k_ in [k_ for k_, v_ in _mask_cache.items() if v_[0]() is None]:
+            del _mask_cache[k_]
+    _mask_cache[key] = (weakref.ref(attn_mask), attn_mask._version, (Sq, Sk), kind, out, compact_kind)
+    return kind, out
+
+
+def _prepare_dropout(dropout_mask, keep_prob):
+    """Returns (uint8 mask or None, keep_prob)."""
+    if dropout_mask is None:
+        return None, 1.0
+    if dropout_mask.dtype in (torch.uint8, torch.bool):
+        d8 = dropout_mask.contiguous()
+        d8 = d8.view(torch.uint8) if d8.dtype == torch.bool else d8
+        if keep_prob is None:
+            raise ValueError("a uint8/bool dropout_mask needs keep_prob")
+        return d8, float(keep_prob)
+    # the reference's form: fp16 {0, 1/keep_prob} (layer/flash_attention.py:198-203)
+    if keep_prob is None:
+        mx = float(dropout_mask.max())
+        keep_prob = 1.0 / mx if mx > 0 else 1.0
+    return dropout_mask.ne(0).to(torch.uint8), float(keep_prob)
+
+
+def _build_params(q, k, v, attn_mask, dropout_mask, alibi_mask, prev_block_num, next_block_num, scale, keep_prob,
+                  row_block_prefix=0):
+    Sq, Sk = q.shape[2], k.shape[2]
+    kind, m8 = (_capi.MASK_NONE, None) if attn_mask is None else _classify_mask(attn_mask, Sq, Sk)
+    if kind == _capi.MASK_CAUSAL and attn_mask is not None and _mask_cache[id(attn_mask)][5] and next_block_num > 0:
+        # a compact tile only ever touches diagonal blocks (attention.py:363-365,
+        # flash_attention_fwd.py:353-356): blocks right of the diagonal stay visible
+        kind, m8 = _capi.MASK_TILE_U8, torch.triu(torch.ones(128, 128, dtype=torch.uint8, device=q.device), diagonal=1)
+    d8, keep = _prepare_dropout(dropout_mask, keep_prob)
+    if alibi_mask is not None and alibi_mask.dtype != q.dtype:
+        alibi_mask = alibi_mask.to(q.dtype)
+    return _capi.make_params(q, k, v, scale=scale, keep_prob=keep, prev_block_num=prev_block_num,
+                             next_block_num=next_block_num, mask_kind=kind, attn_mask=m8, drop_mask=d8,
+                             alibi=alibi_mask, row_block_prefix=row_block_prefix)
+
+
+def _rows_contiguous(t):
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+class _FlashAttentionFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, attn_mask, dropout_mask, alibi_mask, prev_block_num, next_block_num, scale, keep_prob,
+                row_block_prefix):
+        q, k, v = _rows_contiguous(q), _rows_contiguous(k), _rows_contiguous(v)
+        p = _build_params(q, k, v, attn_mask, dropout_mask, alibi_mask, prev_block_num, next_block_num, scale, keep_prob,
+                          row_block_prefix)
+        o, lse = _capi.fa_fwd(p, q)
+        ctx.save_for_backward(q, k, v, o, lse)
+        ctx.params = p
+        ctx.mark_non_differentiable(lse)
+        return o, lse
+
+    @staticmethod
+    def backward(ctx, do, _dlse):
+        q, k, v, o, lse = ctx.saved_tensors
+        dq, dk, dv = _capi.fa_bwd(ctx.params, q, k, v, o, do, lse)
+        return dq, dk, dv, None, None, None, None, None, None, None, None
+
+
+def get_flash_attention_grad(prev_block_num=65536, next_block_num=65536, tiling_stgy_name='sparse',
+                             scale=1.0, keep_prob=None, row_block_prefix=0):
+    """flash_attention_impl.py:96-126 of the reference: returns
+    bprop(query, key, value, attn_mask, dropout_mask, alibi_mask, outs, douts)
+    -> (dq, dk, dv, zeros_like(attn_mask), zeros_like(dropout_mask), zeros_like(alibi_mask))."""
+    _check_strategy(tiling_stgy_name)
+
+    def bprop(query, key, value, attn_mask, dropout_mask, alibi_mask, outs, douts):
+        output, rowsum = outs
+        dout = douts[0]
+        q, k, v = _rows_contiguous(query), _rows_contiguous(key), _rows_contiguous(value)
+        p = _build_params(q, k, v, attn_mask, dropout_mask, alibi_mask, prev_block_num, next_block_num, scale, keep_prob,
+                          row_block_prefix)
+        dq, dk, dv = _capi.fa_bwd(p, q, k, v, output, dout, rowsum)
+        zeros = tuple(None if t is None else torch.zeros_like(t) for t in (attn_mask, dropout_mask, alibi_mask))
+        return (dq, dk, dv) + zeros
+
+    return bprop
+
+
+def get_flash_attention(prev_block_num=65536, next_block_num=65536, tiling_stgy_name='sparse',
+                        scale=1.0, keep_prob=None, row_block_prefix=0):
+    """flash_attention_impl.py:129-154 of the reference: returns the forward
+    primitive (query, key, value, attn_mask=None, dropout_mask=None,
+    alibi_mask=None) -> (output [B,N,Sq,D] in q's dtype, rowsum fp32 [B,N,Sq]),
+    differentiable in query, key and value."""
+    _check_strategy(tiling_stgy_name)
+
+    def fa_forward(query, key, value, attn_mask=None, dropout_mask=None, alibi_mask=None):
+        return _FlashAttentionFn.apply(query, key, value, attn_mask, dropout_mask, alibi_mask,
+                                       prev_block_num, next_block_num, scale, keep_prob, row_block_prefix)
+
+    fa_forward.prev_block_num = prev_block_num
+    fa_forward.next_block_num = next_block_num
+    fa_forward.tiling_stgy_name = tiling_stgy_name
+    fa_forward.bprop = get_flash_attention_grad(prev_block_num, next_block_num, tiling_stgy_name, scale, keep_prob,
+                                                row_block_prefix)
+    return fa_forward

@@ -71,7 +71,9 @@ typedef struct acct_fa_params {
   int32_t prev_block_num;        /* band, in 128-row blocks (T/attention.py:162-167) */
   int32_t next_block_num;        /* 0 = causal block skip */
   int32_t mask_kind;             /* ACCT_MASK_* */
-  int32_t reserved0;
+  int32_t row_block_prefix;      /* 0 = off; else a multiple of 128: query row i sees only keys
+                                    j < (i / row_block_prefix + 1) * row_block_prefix -- the row-block prefixes of
+                                    train/acctransformer/triangle_attention/triangle_attention.py:137-165 */
   int64_t mask_stride_b;         /* elements between batches of attn_mask; 0 = broadcast [1,Sq,Sk] */
   int64_t alibi_stride_b;        /* alibi element strides; stride_q = 0 is the reference's   */
   int64_t alibi_stride_h;        /* [B,N,1,Sk] row-bias form (L/flash_attention.py:185);      */
