@@ -174,12 +174,14 @@ int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, s
   return ACCT_OK;
 }
 
-int acct_fa_bwd(const acct_fa_params* p, const void* O, const void* dO, const float* LSE, void* dQ, void* dK, void* dV,
-                void* workspace, size_t workspace_bytes, void* stream) {
+static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, const float* LSE, void* dQ, void* dK, void* dV,
+                    void* workspace, size_t workspace_bytes, void* stream, int stages) {
   g_err[0] = 0;
   int rc = validate(p);
   if (rc) return rc;
-  if (!O || !dO || !LSE || !dQ || !dK || !dV) return fail(ACCT_E_NULLPTR, "O, dO, LSE, dQ, dK and dV must be non-NULL");
+  const bool want_dq = stages & acct::kStageDq, want_dkdv = stages & acct::kStageDkDv;
+  if (!O || !dO || !LSE || (want_dq && !dQ) || (want_dkdv && (!dK || !dV)))
+    return fail(ACCT_E_NULLPTR, "O, dO, LSE and the requested gradients must be non-NULL");
   if (((uintptr_t)O | (uintptr_t)dO | (uintptr_t)dQ | (uintptr_t)dK | (uintptr_t)dV) & 15)
     return fail(ACCT_E_SHAPE, "O, dO, dQ, dK and dV must be 16-byte aligned");
   if (p->keep_prob < 1.f && !p->drop_mask) return fail(ACCT_E_NULLPTR, "keep_prob < 1 needs a drop_mask");
@@ -198,12 +200,29 @@ int acct_fa_bwd(const acct_fa_params* p, const void* O, const void* dO, const fl
   if (p->mask_kind == ACCT_MASK_DENSE_U8) {
     uint8_t* flags = (uint8_t*)workspace + align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256);
     a.blkflags = flags;
-    hipError_t e = acct::launch_mask_blocks(a, flags, p->mask_stride_b ? p->B : 1, st);
-    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
+    if (want_dq || stages == acct::kStageDkDv) {   // the dkdv-only call re-derives the flags: the mask may have been edited since
+      hipError_t e = acct::launch_mask_blocks(a, flags, p->mask_stride_b ? p->B : 1, st);
+      if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
+    }
   }
-  hipError_t e = acct::launch_bwd(a, p->dtype, p->D, st);
+  hipError_t e = acct::launch_bwd(a, p->dtype, p->D, stages, st);
   if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "backward kernels: %s", hipGetErrorString(e));
   return ACCT_OK;
+}
+
+int acct_fa_bwd(const acct_fa_params* p, const void* O, const void* dO, const float* LSE, void* dQ, void* dK, void* dV,
+                void* workspace, size_t workspace_bytes, void* stream) {
+  return bwd_impl(p, O, dO, LSE, dQ, dK, dV, workspace, workspace_bytes, stream, acct::kStageDq | acct::kStageDkDv);
+}
+
+int acct_fa_bwd_dq(const acct_fa_params* p, const void* O, const void* dO, const float* LSE, void* dQ,
+                   void* workspace, size_t workspace_bytes, void* stream) {
+  return bwd_impl(p, O, dO, LSE, dQ, nullptr, nullptr, workspace, workspace_bytes, stream, acct::kStageDq);
+}
+
+int acct_fa_bwd_dkdv(const acct_fa_params* p, const void* O, const void* dO, const float* LSE, void* dK, void* dV,
+                     void* workspace, size_t workspace_bytes, void* stream) {
+  return bwd_impl(p, O, dO, LSE, nullptr, dK, dV, workspace, workspace_bytes, stream, acct::kStageDkDv);
 }
 
 }  // extern "C"

@@ -469,11 +469,11 @@ __global__ void __launch_bounds__(256) fa_bwd_dkdv_kernel(const FaArgs a) {
 
 // ---- launchers ----------------------------------------------------------------
 template <typename T, int D, bool BIAS, bool DROP>
-static hipError_t launch_bwd_t(FaArgs a, hipStream_t st) {
+static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
   using C = TileCfg<D>;
   const size_t smem = 4 * (size_t)C::TILEB;
-  hipError_t e;
-  {
+  hipError_t e = hipSuccess;
+  if (stages & kStageDq) {
     constexpr int QG = 1;
     a.n_tiles = (a.Sq + 128 * QG - 1) / (128 * QG);
     auto kern = fa_bwd_dq_kernel<T, D, QG, BIAS, DROP>;
@@ -483,7 +483,7 @@ static hipError_t launch_bwd_t(FaArgs a, hipStream_t st) {
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
-  {
+  if (stages & kStageDkDv) {
     constexpr int KG = 1;
     a.n_tiles = (a.Sk + 128 * KG - 1) / (128 * KG);
     auto kern = fa_bwd_dkdv_kernel<T, D, KG, BIAS, DROP>;
@@ -496,21 +496,21 @@ static hipError_t launch_bwd_t(FaArgs a, hipStream_t st) {
 }
 
 template <typename T, int D>
-static hipError_t launch_bwd_d(const FaArgs& a, hipStream_t st) {
+static hipError_t launch_bwd_d(const FaArgs& a, int stages, hipStream_t st) {
   const bool bias = a.alibi != nullptr, drop = a.drop != nullptr;
-  if (bias) return drop ? launch_bwd_t<T, D, true, true>(a, st) : launch_bwd_t<T, D, true, false>(a, st);
-  return drop ? launch_bwd_t<T, D, false, true>(a, st) : launch_bwd_t<T, D, false, false>(a, st);
+  if (bias) return drop ? launch_bwd_t<T, D, true, true>(a, stages, st) : launch_bwd_t<T, D, true, false>(a, stages, st);
+  return drop ? launch_bwd_t<T, D, false, true>(a, stages, st) : launch_bwd_t<T, D, false, false>(a, stages, st);
 }
 
-hipError_t launch_bwd(const FaArgs& a, int dtype, int D, hipStream_t st) {
+hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t st) {
   if (dtype == 0) {
-    if (D == 128) return launch_bwd_d<f16, 128>(a, st);
-    if (D == 64) return launch_bwd_d<f16, 64>(a, st);
-    if (D == 80) return launch_bwd_d<f16, 80>(a, st);
+    if (D == 128) return launch_bwd_d<f16, 128>(a, stages, st);
+    if (D == 64) return launch_bwd_d<f16, 64>(a, stages, st);
+    if (D == 80) return launch_bwd_d<f16, 80>(a, stages, st);
   } else {
-    if (D == 128) return launch_bwd_d<bf16, 128>(a, st);
-    if (D == 64) return launch_bwd_d<bf16, 64>(a, st);
-    if (D == 80) return launch_bwd_d<bf16, 80>(a, st);
+    if (D == 128) return launch_bwd_d<bf16, 128>(a, stages, st);
+    if (D == 64) return launch_bwd_d<bf16, 64>(a, stages, st);
+    if (D == 80) return launch_bwd_d<bf16, 80>(a, stages, st);
   }
   return hipErrorInvalidValue;
 }

@@ -9,7 +9,8 @@ namespace acct {
 hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st);
 
 // backward: delta pre-pass, dK/dV kernel (kv-tile owner) and dQ kernel (q-tile owner)
-hipError_t launch_bwd(const FaArgs& a, int dtype, int D, hipStream_t st);
+enum : int { kStageDq = 1, kStageDkDv = 2 };
+hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t st);
 
 // classify the 128x128 blocks of a dense uint8 mask into clean / apply / skip
 hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, int MB, hipStream_t st);

@@ -108,6 +108,18 @@ int acct_fa_bwd(const acct_fa_params* p, const void* O, const void* dO, const fl
                 void* workspace, size_t workspace_bytes, void* stream);
 size_t acct_fa_bwd_workspace_bytes(const acct_fa_params* p);
 
+/* The two halves of acct_fa_bwd, for callers that need one side of the gradient
+ * only or want to time the halves apart (same workspace size as acct_fa_bwd).
+ * acct_fa_bwd_dq writes dQ (T/flash_attention_bwd.py:209-231) and leaves
+ * D = rowsum(dO*O) (T/flash_attention_bwd.py:138-159) in the workspace;
+ * acct_fa_bwd_dkdv writes dV and dK (T/flash_attention_bwd.py:183-207,233-257)
+ * and reads that D: it must follow an acct_fa_bwd_dq or acct_fa_bwd call with
+ * the same inputs and workspace, in stream order. */
+int acct_fa_bwd_dq(const acct_fa_params* p, const void* O, const void* dO, const float* LSE,
+                   void* dQ, void* workspace, size_t workspace_bytes, void* stream);
+int acct_fa_bwd_dkdv(const acct_fa_params* p, const void* O, const void* dO, const float* LSE,
+                     void* dK, void* dV, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Thread-local text of the last error on the calling thread ("" if none).
  * Stands in for the Python exceptions the reference raises at build time
  * (L/flash_attention.py:105-108,193-196). */

@@ -222,11 +222,16 @@ def unfused_fwd(q, k, v, scale=1.0, attn_mask=None, alibi=None, drop_mask=None, 
 
 
 def unfused_bwd(q, k, v, dO, scale=1.0, attn_mask=None, alibi=None, drop_mask=None, keep_prob=1.0,
-                prev_block_num=BLOCK_NUM_UNBOUNDED, next_block_num=BLOCK_NUM_UNBOUNDED):
+                prev_block_num=BLOCK_NUM_UNBOUNDED, next_block_num=BLOCK_NUM_UNBOUNDED, O_saved=None):
     """Analytic gradient of unfused_fwd in fp64 (T/flash_attention_bwd.py:88-257):
 
       P = softmax(S) ; Pd = P*drop/keep ; dV = Pd^T dO ; dP = (dO v^T)*drop/keep
       D = rowsum(dO * O) ; dS = P*(dP - D) ; dQ = scale dS k ; dK = scale dS^T q
+
+    With O_saved (the forward's rounded output) D is taken from it instead of
+    the exact O: the "fa version" ground truth of ST/common.py:156-169, which
+    the reference adopts because the rounding of the saved O otherwise
+    dominates the comparison when the softmax is nearly one-hot.
     """
     B, N, Sq, D = q.shape
     Sk = k.shape[2]
@@ -245,7 +250,7 @@ def unfused_bwd(q, k, v, dO, scale=1.0, attn_mask=None, alibi=None, drop_mask=No
             pd = p if dr is None else p * dr
             do = dO[b, h].astype(np.float64)
             vv = v[b, h].astype(np.float64)
-            o = pd @ vv
+            o = pd @ vv if O_saved is None else np.asarray(O_saved[b, h], dtype=np.float64)
             dV[b, h] = pd.T @ do
             dp = do @ vv.T
             if dr is not None:

@@ -1,0 +1,177 @@
+"""CPU-side tests: the C-ABI library loads and exports what include/acct_fa.h
+declares, argument validation returns the documented error codes without
+touching a device, and the Python mirror of the reference interface keeps the
+reference's names, argument checks and error texts."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from acctransformer_amd import _capi
+from acctransformer_amd.flash_attention.nn.layer.flash_attention import FlashAttention
+from acctransformer_amd.flash_attention.ops.flash_attention import flash_attention_impl as impl
+from acctransformer_amd.triangle_attention.triangle_attention import TriangleAttention
+from golden_cases import load_cases
+from oracle import unfused_attention as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header():
+    return open(os.path.join(ROOT, "include", "acct_fa.h")).read()
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _capi.load()
+    decl = re.findall(r"^\s*(?:int|size_t|const char\*)\s+(acct_\w+)\s*\(", _header(), flags=re.M)
+    assert set(decl) >= {"acct_fa_fwd", "acct_fa_bwd", "acct_fa_bwd_dq", "acct_fa_bwd_dkdv",
+                         "acct_fa_fwd_workspace_bytes", "acct_fa_bwd_workspace_bytes", "acct_last_error", "acct_version"}
+    for name in decl:
+        assert hasattr(lib, name), name
+    m = re.search(r"#define ACCT_FA_VERSION (\d+)", _header())
+    assert lib.acct_version() == int(m.group(1))
+
+
+def test_struct_mirror_matches_header_field_order():
+    body = re.search(r"typedef struct acct_fa_params \{(.*?)\} acct_fa_params;", _header(), flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    names = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        for part in decl.split(","):
+            names.append(re.sub(r"\[\d+\]", "", part.strip().split()[-1]).lstrip("*"))
+    assert names == [f[0] for f in _capi.AcctFaParams._fields_]
+    assert ctypes.sizeof(_capi.AcctFaParams) == 224
+
+
+def _params(**over):
+    q = torch.zeros(1, 2, 128, 128, dtype=torch.float16)
+    p = _capi.make_params(q, q.clone(), q.clone(), scale=1.0)
+    for k, v in over.items():
+        setattr(p, k, v)
+    return p
+
+
+@pytest.mark.parametrize("over, code", [
+    (dict(dtype=7), -3), (dict(B=0), -2), (dict(D=512), -4), (dict(D=96), -4), (dict(scale=0.0), -8),
+    (dict(keep_prob=1.5), -8), (dict(prev_block_num=-1), -8), (dict(mask_kind=2), -8),
+    (dict(mask_kind=_capi.MASK_DENSE_U8), -1), (dict(row_block_prefix=100), -8), (dict(q=None), -1),
+])
+def test_validation_error_codes(over, code):
+    lib = _capi.load()
+    p = _params(**over)
+    buf = (ctypes.c_char * 64)()
+    rc = lib.acct_fa_fwd(ctypes.byref(p), ctypes.addressof(buf), ctypes.addressof(buf), None, 0, None)
+    assert rc == code
+    assert lib.acct_last_error().decode() != ""
+    rc = lib.acct_fa_bwd(ctypes.byref(p), *([ctypes.addressof(buf)] * 6), None, 0, None)
+    assert rc == code
+
+
+def test_null_outputs_and_workspace_sizes():
+    lib = _capi.load()
+    p = _params()
+    assert lib.acct_fa_fwd(ctypes.byref(p), None, None, None, 0, None) == -1
+    assert lib.acct_fa_fwd(None, None, None, None, 0, None) == -1
+    assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p)) == 0
+    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p)) == 1 * 2 * 128 * 4
+    m = torch.zeros(1, 128, 128, dtype=torch.uint8)
+    q = torch.zeros(2, 2, 128, 128, dtype=torch.float16)
+    p2 = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m)
+    assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p2)) == 256
+    raw = (ctypes.c_char * 128)()
+    addr = (ctypes.addressof(raw) + 63) // 64 * 64
+    # backward without its workspace is refused before any launch
+    assert lib.acct_fa_bwd(ctypes.byref(p2), *([addr] * 6), None, 0, None) == -7
+    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p2)) == 2 * 2 * 128 * 4 + 256
+
+
+def test_no_cpu_fallback():
+    q = torch.zeros(1, 1, 128, 64, dtype=torch.float16)
+    p = _capi.make_params(q, q.clone(), q.clone(), scale=1.0)
+    with pytest.raises(RuntimeError):
+        _capi.fa_fwd(p, q)
+
+
+# ---- the Python mirror of the reference interface -------------------------------
+def test_layer_constructor_checks_match_reference():
+    with pytest.raises(ValueError, match="head_dim too large"):
+        FlashAttention(head_dim=512)
+    with pytest.raises(ValueError, match="alibi not supported"):
+        FlashAttention(head_dim=128, alibi=True)
+    with pytest.raises(Exception, match="Strategy:foo not supported"):
+        FlashAttention(head_dim=128, tiling_stgy_name="foo")
+    layer = FlashAttention(head_dim=128, dropout_rate=0.1, prev_block_num=7, next_block_num=0)
+    assert np.isclose(layer.scale, orc.flash_attention_layer_scale(128))
+    assert layer.shard(((2, 4, 1, 1),) * 3) is layer and (layer.dp, layer.mp) == (2, 4)
+    q = torch.zeros(1, 2, 128, 128, dtype=torch.float16)
+    k = torch.zeros(1, 3, 128, 128, dtype=torch.float16)
+    with pytest.raises(ValueError, match="head_num of query, key and value must be the same"):
+        layer(q, k, k)
+
+
+def test_triangle_constructor_checks_match_reference():
+    with pytest.raises(ValueError, match="block size must be positive"):
+        TriangleAttention(block_size=0)
+    with pytest.raises(ValueError, match="dropout rate must be between 0 and 1"):
+        TriangleAttention(dropout_rate=1.0)
+    with pytest.raises(ValueError, match="data parallel must be positive"):
+        TriangleAttention(dp=0)
+    with pytest.raises(ValueError, match="model parallel must be positive"):
+        TriangleAttention(mp=-1)
+    assert TriangleAttention().block_size == 512
+
+
+def test_op_factories_keep_reference_signature():
+    fwd = impl.get_flash_attention(prev_block_num=3, next_block_num=0, tiling_stgy_name="wukong")
+    assert (fwd.prev_block_num, fwd.next_block_num, fwd.tiling_stgy_name) == (3, 0, "wukong")
+    assert callable(impl.get_flash_attention_grad())
+    with pytest.raises(Exception, match="not supported"):
+        impl.get_flash_attention(tiling_stgy_name="nope")
+
+
+def test_mask_classification():
+    S = 256
+    tri = torch.triu(torch.ones(1, S, S, dtype=torch.float16), 1)
+    assert impl._classify_mask(tri, S, S)[0] == _capi.MASK_CAUSAL
+    pad = torch.zeros(2, S, S, dtype=torch.uint8); pad[:, :, 200:] = 1
+    kind, m8 = impl._classify_mask(pad, S, S)
+    assert kind == _capi.MASK_DENSE_U8 and m8.dtype == torch.uint8 and m8.shape == (2, S, S)
+    tile = torch.triu(torch.ones(1, 128, 128, dtype=torch.float16), 1)
+    assert impl._classify_mask(tile, S, S)[0] == _capi.MASK_CAUSAL
+    odd = tile.clone(); odd[0, 5, 3] = 1
+    kind, m8 = impl._classify_mask(odd, S, S)
+    assert kind == _capi.MASK_TILE_U8 and m8.shape == (128, 128)
+    # remembered per tensor and version: an in-place edit is seen
+    tri[0, 0, 1] = 0
+    assert impl._classify_mask(tri, S, S)[0] == _capi.MASK_DENSE_U8
+    with pytest.raises(ValueError):
+        impl._classify_mask(torch.zeros(1, 100, S), S, S)
+
+
+def test_dropout_mask_forms():
+    d = torch.tensor([[0.0, 1.25], [1.25, 0.0]], dtype=torch.float16)
+    m8, keep = impl._prepare_dropout(d, None)
+    assert m8.tolist() == [[0, 1], [1, 0]] and np.isclose(keep, 0.8)
+    m8, keep = impl._prepare_dropout(torch.tensor([[1, 0]], dtype=torch.uint8), 0.9)
+    assert keep == 0.9
+    with pytest.raises(ValueError):
+        impl._prepare_dropout(torch.tensor([[1, 0]], dtype=torch.uint8), None)
+
+
+# ---- the oracle still reproduces the committed fixtures -------------------------
+@pytest.mark.parametrize("name", sorted(load_cases().keys()))
+def test_oracle_reproduces_golden(name):
+    c = load_cases()[name]
+    kw = dict(scale=float(c["scale"]), attn_mask=c.get("attn_mask"), drop_mask=c.get("drop_mask"),
+              alibi=None if "alibi" not in c else c["alibi"].astype(np.float32), keep_prob=float(c["keep_prob"]),
+              prev_block_num=int(c["prev_block_num"]), next_block_num=int(c["next_block_num"]))
+    O, L = orc.unfused_fwd(c["q"], c["k"], c["v"], **kw)
+    dQ, dK, dV = orc.unfused_bwd(c["q"], c["k"], c["v"], c["dO"], **kw)
+    for got, want in ((O, c["O"]), (L, c["L"]), (dQ, c["dQ"]), (dK, c["dK"]), (dV, c["dV"])):
+        assert np.allclose(got, want, rtol=1e-6, atol=1e-6)
