@@ -1,0 +1,196 @@
+"""Benchmark of the FlashAttention2 forward + backward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one forward call and one backward call of the attention operator
+through the C ABI, on the workload BASELINE.json quotes its metric on:
+B=4, N=16, S=2048, D=128, fp16, causal attn_mask (uint8, 1 = masked),
+keep_prob = 1, upstream dO ~ N(0,1).  Inputs are synthetic and already resident
+in HBM.  Prints one JSON line: whole-job TFLOP/s by the FlashAttention-2 flop
+convention (fwd 4*B*N*S^2*D*f, bwd 2.5x, f = 1/2 causal), the roofline of the
+dominant kernel from HIP-event timings taken inside the timed region, and the
+CPU baseline (the reference's numpy unfused attention, restated in oracle/,
+timed on this box's host cores on its own CPU-sized configuration).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2516.6          # MI355X dense fp16 MFMA peak (256 CU x 4 SIMD x 1024 flop/clk x 2.4 GHz)
+
+
+def cpu_baseline(budget_s=12.0):
+    """The reference's CPU attention path (tests/train/flash_attention/st/common.py:110-132,
+    restated in oracle/unfused_attention.py) on its CPU-runnable configuration:
+    B=1, N=4, S=512, D=64, fp16 N(0,1), scale 1/8 folded into q, no mask, forward only."""
+    import numpy as np
+    import torch
+    from oracle import unfused_attention as orc
+    rng = np.random.default_rng(1000)
+    q, k, v = (rng.standard_normal((1, 4, 512, 64)).astype(np.float16) for _ in range(3))
+    qs = (q.astype(np.float32) * 0.125).astype(np.float16)
+    flops = 4 * 1 * 4 * 512 * 512 * 64
+    orc.np_unfused_fwd_fp16(qs, k, v)
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while time.perf_counter() < t_end and len(times) < 50:
+        t0 = time.perf_counter()
+        orc.np_unfused_fwd_fp16(qs, k, v)
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    # second formulation: torch fp32 on all host cores (tests/infer/flash_attention/tik/data_gen.py:32-34)
+    threads = min(16, os.cpu_count() or 1)
+    torch.set_num_threads(threads)
+    tq, tk, tv = (torch.from_numpy(x) for x in (qs, k, v))
+    for _ in range(3):
+        orc.torch_unfused_fwd_fp32(tq, tk, tv)
+    tt = []
+    for _ in range(20):
+        t0 = time.perf_counter()
+        orc.torch_unfused_fwd_fp32(tq, tk, tv)
+        tt.append(time.perf_counter() - t0)
+    tmed = sorted(tt)[len(tt) // 2]
+    return {
+        "value": flops / med / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+        "sample": f"unfused fwd B1 N4 S512 D64 fp16 (numpy fp16 matmul, the reference's CPU oracle), median of {len(times)} calls, {med * 1e3:.1f} ms/call",
+        "torch_fp32_value": flops / tmed / 1e12, "torch_fp32_cores": threads, "torch_fp32_ms": tmed * 1e3,
+        "host_cpus": os.cpu_count(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures the single-GPU attention hot path: run it with --gpus 1 "
+              "(every (batch, head) pair is independent, so more GPUs would only split B*N; nothing here uses a second GPU)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from acctransformer_amd import _capi
+    from acctransformer_amd.flash_attention.ops.flash_attention import flash_attention_impl as impl
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: the attention path has no CPU fallback", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _capi.load()
+
+    B, N, S, D = 4, 16, 2048, 128
+    g = torch.Generator(device="cpu").manual_seed(1001)
+    q, k, v, dO = (torch.randn(B, N, S, D, generator=g).half().to(dev) for _ in range(4))
+    attn_mask = torch.triu(torch.ones(1, S, S, dtype=torch.uint8, device=dev), 1)
+    scale = D ** -0.5
+    # The operator inspects the mask once per tensor (it is a causal lower-triangular mask: rows are
+    # evaluated by index compare on diagonal tiles, blocks above the diagonal are skipped) ...
+    p = impl._build_params(q, k, v, attn_mask, None, None, 65536, 0, scale, None)
+    # ... and the same workload with the mask read as an arbitrary dense uint8 tensor, for comparison
+    p_dense = _capi.make_params(q, k, v, scale=scale, next_block_num=0, mask_kind=_capi.MASK_DENSE_U8, attn_mask=attn_mask)
+
+    o = torch.empty_like(q)
+    lse = torch.empty(B, N, S, dtype=torch.float32, device=dev)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    for pp in (p, p_dense):
+        pp.o_stride = _capi._bhs_strides(o)
+    nws = max(lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p_dense)), lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p_dense)), 256)
+    ws = torch.empty(nws, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream()
+    st = ctypes.c_void_p(stream.cuda_stream)
+    P = ctypes.byref
+
+    def check(rc):
+        if rc != 0:
+            raise RuntimeError(lib.acct_last_error().decode())
+
+    def fwd(pp):
+        check(lib.acct_fa_fwd(P(pp), o.data_ptr(), lse.data_ptr(), ws.data_ptr(), nws, st))
+
+    def bwd_dq(pp):
+        check(lib.acct_fa_bwd_dq(P(pp), o.data_ptr(), dO.data_ptr(), lse.data_ptr(), dq.data_ptr(), ws.data_ptr(), nws, st))
+
+    def bwd_dkdv(pp):
+        check(lib.acct_fa_bwd_dkdv(P(pp), o.data_ptr(), dO.data_ptr(), lse.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), nws, st))
+
+    def step(pp):
+        fwd(pp); bwd_dq(pp); bwd_dkdv(pp)
+
+    for _ in range(args.warmup):
+        step(p)
+    torch.cuda.synchronize()
+
+    K = args.steps
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(K)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        ev[i][0].record(stream); fwd(p)
+        ev[i][1].record(stream); bwd_dq(p)
+        ev[i][2].record(stream); bwd_dkdv(p)
+        ev[i][3].record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_step = wall * 1e3 / K
+    t_fwd = sum(e[0].elapsed_time(e[1]) for e in ev) / K
+    t_dq = sum(e[1].elapsed_time(e[2]) for e in ev) / K
+    t_dkdv = sum(e[2].elapsed_time(e[3]) for e in ev) / K
+
+    # dense-mask reading of the same workload (untimed for `value`)
+    for _ in range(3):
+        step(p_dense)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for _ in range(K):
+        step(p_dense)
+    torch.cuda.synchronize()
+    ms_dense = (time.perf_counter() - t1) * 1e3 / K
+
+    f = 0.5
+    fl_fwd = 4.0 * B * N * S * S * D * f
+    fl_bwd = 2.5 * fl_fwd
+    fl_step = fl_fwd + fl_bwd
+    value = fl_step / (ms_step * 1e-3) / 1e12
+
+    # dominant kernel: the dK/dV kernel of the backward.  Algorithmic flops per launch: 4 of the 5
+    # backward matmuls (S, dP, dV, dK) = 8*B*N*S^2*D*f; the dQ kernel carries the fifth plus its
+    # own recompute of S and dP.
+    kernels = {
+        "fa_fwd_kernel": (t_fwd, fl_fwd),
+        "fa_bwd_dq_kernel": (t_dq, 0.2 * fl_bwd),
+        "fa_bwd_dkdv_kernel": (t_dkdv, 0.8 * fl_bwd),
+    }
+    dom = max(kernels, key=lambda n: kernels[n][0])
+    dom_ms, dom_fl = kernels[dom]
+    achieved = dom_fl / (dom_ms * 1e-3) / 1e12
+    out = {
+        "metric": "FA2 fwd+bwd TFLOP/s & % fp16 MFMA peak, B4 N16 S2048 D128 causal",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": K, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16", "data": "synthetic",
+        "config": {"workload": "FlashAttention2 fwd+bwd B=4 N=16 S=2048 D=128 fp16, causal uint8 attn_mask, keep_prob=1.0, next_block_num=0",
+                   "flop_convention": "fwd 4*B*N*S^2*D*f, bwd 2.5x fwd, f=0.5", "gflop_per_step": round(fl_step / 1e9, 1)},
+        "pct_of_fp16_mfma_peak": round(100.0 * value / PEAK_FP16_TFLOPS, 2),
+        "kernel_ms": {"fa_fwd_kernel": round(t_fwd, 4), "fa_bwd_dq_kernel": round(t_dq, 4), "fa_bwd_dkdv_kernel": round(t_dkdv, 4)},
+        "fwd_tflops": round(fl_fwd / (t_fwd * 1e-3) / 1e12, 1), "bwd_tflops": round(fl_bwd / ((t_dq + t_dkdv) * 1e-3) / 1e12, 1),
+        "dense_mask_path_ms_per_step": round(ms_dense, 4),
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": None},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
