@@ -166,9 +166,10 @@ int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, s
     hipError_t e = acct::launch_mask_blocks(a, (uint8_t*)workspace, p->mask_stride_b ? p->B : 1, st);
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
   }
-  // 64 query rows per wave (256 per workgroup) once that still fills the chip
-  int qg = ((long long)p->B * p->N * ((p->Sq + 255) / 256) >= n_cu) ? 2 : 1;
-  qg = env_int("ACCT_FA_FWD_QG", qg) == 1 ? 1 : 2;
+  // 8 waves x 32 query rows (two waves per SIMD overlap MFMA and softmax work) once that still
+  // fills the chip, else 4 waves x 32 rows for more workgroups
+  int qg = ((long long)p->B * p->N * ((p->Sq + 255) / 256) >= n_cu) ? 3 : 1;
+  qg = env_int("ACCT_FA_FWD_VARIANT", qg);
   hipError_t e = acct::launch_fwd(a, p->dtype, p->D, qg, st);
   if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "forward kernel: %s", hipGetErrorString(e));
   return ACCT_OK;

@@ -42,14 +42,15 @@ ACCT_DEV typename Elem<T>::V8 pack8(const float* x) {
 // ============================================================================
 // dQ kernel (and delta): query-tile owner, structure of the forward kernel
 // ============================================================================
-template <typename T, int D, int QG, bool BIAS, bool DROP>
-__global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
+template <typename T, int D, int QG, int NW, bool BIAS, bool DROP>
+__global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   using E = Elem<T>;
   using V8 = typename E::V8;
-  using C = TileCfg<D>;
-  constexpr int BM = 128 * QG;
+  using C = SwzCfg<D>;
+  constexpr int BM = 32 * QG * NW;
+  constexpr int TILEB = 64 * C::PITCH;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 buffers][K tile | V tile]
+  ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 buffers][K tile | V tile]; reused by the epilogue
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, g = lane >> 5;
   const int BH = a.B * a.N;
@@ -82,18 +83,13 @@ __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
 #pragma unroll
   for (int gq = 0; gq < QG; gq++) {
     const int row = wq0 + 32 * gq + l32;
+    const int row_c = min(row, a.Sq - 1);
     float part = 0.f;
 #pragma unroll
     for (int t = 0; t < C::KS; t++) {
-      V8 z = {};
-      V8 ov = z;
-      qf[gq][t] = z;
-      dof[gq][t] = z;
-      if (row < a.Sq) {
-        qf[gq][t] = *reinterpret_cast<const V8*>(qp + (int64_t)row * a.q_ss + 16 * t + 8 * g);
-        dof[gq][t] = *reinterpret_cast<const V8*>(dop + (int64_t)row * a.o_ss + 16 * t + 8 * g);
-        ov = *reinterpret_cast<const V8*>(op + (int64_t)row * a.o_ss + 16 * t + 8 * g);
-      }
+      qf[gq][t] = *reinterpret_cast<const V8*>(qp + (int64_t)row_c * a.q_ss + 16 * t + 8 * g);
+      dof[gq][t] = *reinterpret_cast<const V8*>(dop + (int64_t)row_c * a.o_ss + 16 * t + 8 * g);
+      const V8 ov = *reinterpret_cast<const V8*>(op + (int64_t)row_c * a.o_ss + 16 * t + 8 * g);
 #pragma unroll
       for (int e = 0; e < 8; e++) part += (float)dof[gq][t][e] * (float)ov[e];
     }
@@ -104,6 +100,16 @@ __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
       if (g == 0) a.delta[(int64_t)bh * a.Sq + row] = dl[gq];
     }
   }
+
+  // per-lane LDS offsets (tile-invariant)
+  int koff[C::KS];
+#pragma unroll
+  for (int t = 0; t < C::KS; t++) koff[t] = l32 * C::PITCH + swz_off(2 * t + g, l32 & 7);
+  const int trow = 4 * g + ((lane & 15) >> 2);
+  const int tchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+  int toff[C::DB];
+#pragma unroll
+  for (int db = 0; db < C::DB; db++) toff[db] = trow * C::PITCH + swz_off(4 * db + tchunk, trow) + 8 * (lane & 1);
 
   f32x16 acc[QG][C::DB];
 #pragma unroll
@@ -123,21 +129,18 @@ __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
   const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
   if (j_lo <= j_hi) {
-    u32x4 kreg[C::NLD], vreg[C::NLD];
-    tile_load<T, D>(kp, a.k_ss, j_lo * 64, a.Sk, kreg);
-    tile_load<T, D>(vp, a.v_ss, j_lo * 64, a.Sk, vreg);
-    tile_store<D>(smem, kreg);
-    tile_store<D>(smem + C::TILEB, vreg);
+    tile_dma<T, D, 64, NW>(kp, a.k_ss, j_lo * 64, a.Sk, smem);
+    tile_dma<T, D, 64, NW>(vp, a.v_ss, j_lo * 64, a.Sk, smem + TILEB);
+    dma_wait();
     __syncthreads();
 
     for (int j = j_lo; j <= j_hi; j++) {
       const int buf = (j - j_lo) & 1;
-      ACCT_LDS char* kbuf = smem + buf * 2 * C::TILEB;
-      ACCT_LDS char* vbuf = kbuf + C::TILEB;
-      const bool more = j < j_hi;
-      if (more) {
-        tile_load<T, D>(kp, a.k_ss, (j + 1) * 64, a.Sk, kreg);
-        tile_load<T, D>(vp, a.v_ss, (j + 1) * 64, a.Sk, vreg);
+      ACCT_LDS char* kbuf = smem + buf * 2 * TILEB;
+      ACCT_LDS char* vbuf = kbuf + TILEB;
+      if (j < j_hi) {
+        tile_dma<T, D, 64, NW>(kp, a.k_ss, (j + 1) * 64, a.Sk, smem + (buf ^ 1) * 2 * TILEB);
+        tile_dma<T, D, 64, NW>(vp, a.v_ss, (j + 1) * 64, a.Sk, smem + (buf ^ 1) * 2 * TILEB + TILEB);
       }
       const int kv0 = j * 64;
       const int kvb = j >> 1;
@@ -152,8 +155,7 @@ __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
       } else if (a.mask_kind == kMaskTile) {
         apply_mask = wqb == kvb;
       }
-      const bool diag = causal && (kv0 + 63 > wq0);
-      const bool tail = kv0 + 64 > a.Sk;
+      const bool edge = apply_mask || (causal && (kv0 + 63 > wq0)) || (kv0 + 64 > a.Sk);
       if (act) {
         V8 dsf[QG][2][2];
 #pragma unroll
@@ -163,15 +165,20 @@ __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
           for (int gq = 0; gq < QG; gq++)
 #pragma unroll
             for (int r = 0; r < 16; r++) { s[gq][r] = 0.f; dp[gq][r] = 0.f; }
+          {
+            V8 kf[C::KS], vf[C::KS];
 #pragma unroll
-          for (int t = 0; t < C::KS; t++) {
-            const V8 kf = lds_read_frag<T>(kbuf + (32 * c + l32) * C::ROWB + (16 * t + 8 * g) * 2);
-            const V8 vf = lds_read_frag<T>(vbuf + (32 * c + l32) * C::ROWB + (16 * t + 8 * g) * 2);
+            for (int t = 0; t < C::KS; t++) kf[t] = lds_read_frag<T>(kbuf + koff[t] + c * 32 * C::PITCH);
 #pragma unroll
-            for (int gq = 0; gq < QG; gq++) {
-              s[gq] = E::mfma(kf, qf[gq][t], s[gq]);
-              dp[gq] = E::mfma(vf, dof[gq][t], dp[gq]);
-            }
+            for (int t = 0; t < C::KS; t++) vf[t] = lds_read_frag<T>(vbuf + koff[t] + c * 32 * C::PITCH);
+#pragma unroll
+            for (int t = 0; t < C::KS; t++)
+#pragma unroll
+              for (int gq = 0; gq < QG; gq++) s[gq] = E::mfma(kf[t], qf[gq][t], s[gq]);
+#pragma unroll
+            for (int t = 0; t < C::KS; t++)
+#pragma unroll
+              for (int gq = 0; gq < QG; gq++) dp[gq] = E::mfma(vf[t], dof[gq][t], dp[gq]);
           }
           // element (gq, r): q = wq0 + 32 gq + l32 ; kv = kv0 + 32 c + 8 (r/4) + 4 g + r%4
 #pragma unroll
@@ -179,30 +186,36 @@ __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
             const int qrow = wq0 + 32 * gq + l32;
             const int qrow_c = min(qrow, a.Sq - 1);
             float ds[16];
+            if (!edge && !BIAS && !DROP) {                   // interior tile: no side inputs at all
 #pragma unroll
-            for (int r4 = 0; r4 < 4; r4++) {
-              const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
-              float bias[4] = {0.f, 0.f, 0.f, 0.f};
-              uint32_t mbits = 0, dbits = 0x01010101u;
-              if (BIAS) load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
-              if (apply_mask) {
-                if (a.mask_kind == kMaskDense) mbits = load_u8x4(maskp + (int64_t)qrow_c * a.Sk, kv, a.Sk, mask_vec);
-                else mbits = load_u8x4(maskp + (qrow_c & 127) * 128, kv & 127, 128, mask_vec);
+              for (int r = 0; r < 16; r++) {
+                const float p = fast_exp2(__builtin_fmaf(s[gq][r], a.scale_log2e, -lq[gq]));
+                ds[r] = p * (dp[gq][r] - dl[gq]);
               }
-              if (DROP) dbits = load_u8x4(dropp + (int64_t)qrow_c * a.Sk, kv, a.Sk, drop_vec);
+            } else {
 #pragma unroll
-              for (int e = 0; e < 4; e++) {
-                const int r = 4 * r4 + e;
-                float x = __builtin_fmaf(s[gq][r], a.scale_log2e, -lq[gq]);
-                if (BIAS) x = __builtin_fmaf(bias[e], kLog2e, x);
-                if (apply_mask || diag) {
-                  if (((mbits >> (8 * e)) & 0xffu) || (causal && kv + e > qrow)) x += kMaskFill * kLog2e;
+              for (int r4 = 0; r4 < 4; r4++) {
+                const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
+                float bias[4] = {0.f, 0.f, 0.f, 0.f};
+                uint32_t mbits = 0, dbits = 0x01010101u;
+                if (BIAS) load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
+                if (apply_mask) {
+                  if (a.mask_kind == kMaskDense) mbits = load_u8x4(maskp + (int64_t)qrow_c * a.Sk, kv, a.Sk, mask_vec);
+                  else mbits = load_u8x4(maskp + (qrow_c & 127) * 128, kv & 127, 128, mask_vec);
                 }
-                float p = fast_exp2(x);
-                if (tail && kv + e >= a.Sk) p = 0.f;
-                float dpv = dp[gq][r];
-                if (DROP) dpv = ((dbits >> (8 * e)) & 0xffu) ? dpv * a.inv_keep : 0.f;
-                ds[r] = p * (dpv - dl[gq]);
+                if (DROP) dbits = load_u8x4(dropp + (int64_t)qrow_c * a.Sk, kv, a.Sk, drop_vec);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                  const int r = 4 * r4 + e;
+                  float x = __builtin_fmaf(s[gq][r], a.scale_log2e, -lq[gq]);
+                  if (BIAS) x = __builtin_fmaf(bias[e], kLog2e, x);
+                  if (((mbits >> (8 * e)) & 0xffu) || (causal && kv + e > qrow)) x += kMaskFill * kLog2e;
+                  float p = fast_exp2(x);
+                  if (kv + e >= a.Sk) p = 0.f;
+                  float dpv = dp[gq][r];
+                  if (DROP) dpv = ((dbits >> (8 * e)) & 0xffu) ? dpv * a.inv_keep : 0.f;
+                  ds[r] = p * (dpv - dl[gq]);
+                }
               }
             }
             dsf[gq][c][0] = pack8<T>(ds);
@@ -216,40 +229,42 @@ __global__ void __launch_bounds__(256) fa_bwd_dq_kernel(const FaArgs a) {
           for (int hh = 0; hh < 2; hh++)
 #pragma unroll
             for (int db = 0; db < C::DB; db++) {
-              const ACCT_LDS char* kaddr = kbuf + (32 * c + 16 * hh + 4 * g + ((lane & 15) >> 2)) * C::ROWB +
-                                           (32 * db + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
-              const V8 ktf = join_tr<T>(lds_read_tr(kaddr), lds_read_tr(kaddr + 8 * C::ROWB));
+              const ACCT_LDS char* kaddr = kbuf + toff[db] + (32 * c + 16 * hh) * C::PITCH;
+              const V8 ktf = join_tr<T>(lds_read_tr(kaddr), lds_read_tr(kaddr + 8 * C::PITCH));
 #pragma unroll
               for (int gq = 0; gq < QG; gq++) acc[gq][db] = E::mfma(ktf, dsf[gq][c][hh], acc[gq][db]);
             }
       }
-      if (more) {
-        ACCT_LDS char* nk = smem + (buf ^ 1) * 2 * C::TILEB;
-        tile_store<D>(nk, kreg);
-        tile_store<D>(nk + C::TILEB, vreg);
-      }
+      dma_wait();
       __syncthreads();
     }
   }
 
-  // ---- epilogue: dQ = scale * dQ^T ----
+  // ---- epilogue: dQ = scale * dQ^T, transposed through the wave's own LDS region ----
   T* dqp = (T*)a.dq + b * a.q_sb + h * a.q_sh;
+  constexpr int OPITCH = C::DB * 64 + 16;
+  ACCT_LDS char* obuf = smem + wave * (32 * OPITCH);
 #pragma unroll
   for (int gq = 0; gq < QG; gq++) {
-    const int row = wq0 + 32 * gq + l32;
-    if (row < a.Sq) {
 #pragma unroll
-      for (int db = 0; db < C::DB; db++)
+    for (int db = 0; db < C::DB; db++)
 #pragma unroll
-        for (int r4 = 0; r4 < 4; r4++) {
-          const int d = 32 * db + 8 * r4 + 4 * g;
-          if (d < D) {
-            typename E::V2 t0 = E::cvt2(acc[gq][db][4 * r4 + 0] * a.scale, acc[gq][db][4 * r4 + 1] * a.scale);
-            typename E::V2 t1 = E::cvt2(acc[gq][db][4 * r4 + 2] * a.scale, acc[gq][db][4 * r4 + 3] * a.scale);
-            typename E::V4 ov = {t0[0], t0[1], t1[0], t1[1]};
-            *reinterpret_cast<typename E::V4*>(dqp + (int64_t)row * a.q_ss + d) = ov;
-          }
-        }
+      for (int r4 = 0; r4 < 4; r4++) {
+        typename E::V2 t0 = E::cvt2(acc[gq][db][4 * r4 + 0] * a.scale, acc[gq][db][4 * r4 + 1] * a.scale);
+        typename E::V2 t1 = E::cvt2(acc[gq][db][4 * r4 + 2] * a.scale, acc[gq][db][4 * r4 + 3] * a.scale);
+        typename E::V4 ov = {t0[0], t0[1], t1[0], t1[1]};
+        *reinterpret_cast<ACCT_LDS typename E::V4*>(obuf + l32 * OPITCH + (32 * db + 8 * r4 + 4 * g) * 2) = ov;
+      }
+    constexpr int NCH = C::CPR;
+#pragma unroll
+    for (int i = 0; i < (32 * NCH + 63) / 64; i++) {
+      const int idx = lane + 64 * i;
+      const int r = idx / NCH, ch = idx % NCH;
+      const int grow = wq0 + 32 * gq + r;
+      if (idx < 32 * NCH && grow < a.Sq) {
+        const u32x4 v = *reinterpret_cast<const ACCT_LDS u32x4*>(obuf + r * OPITCH + ch * 16);
+        *reinterpret_cast<u32x4*>(dqp + (int64_t)grow * a.q_ss + ch * 8) = v;
+      }
     }
   }
 }
@@ -474,12 +489,16 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
   const size_t smem = 4 * (size_t)C::TILEB;
   hipError_t e = hipSuccess;
   if (stages & kStageDq) {
-    constexpr int QG = 1;
-    a.n_tiles = (a.Sq + 128 * QG - 1) / (128 * QG);
-    auto kern = fa_bwd_dq_kernel<T, D, QG, BIAS, DROP>;
+    constexpr int QG = 1, NW = 8;
+    constexpr int BM = 32 * QG * NW;
+    using CS = SwzCfg<D>;
+    constexpr size_t tiles = 4 * 64 * (size_t)CS::PITCH, stage = (size_t)NW * 32 * (CS::DB * 64 + 16);
+    const size_t smem = tiles > stage ? tiles : stage;
+    a.n_tiles = (a.Sq + BM - 1) / BM;
+    auto kern = fa_bwd_dq_kernel<T, D, QG, NW, BIAS, DROP>;
     e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((unsigned)((long long)a.n_tiles * a.B * a.N)), dim3(256), smem, st, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((long long)a.n_tiles * a.B * a.N)), dim3(64 * NW), smem, st, a);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -498,11 +517,17 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
 template <typename T, int D>
 static hipError_t launch_bwd_d(const FaArgs& a, int stages, hipStream_t st) {
   const bool bias = a.alibi != nullptr, drop = a.drop != nullptr;
+#ifndef ACCT_DEV_BUILD
   if (bias) return drop ? launch_bwd_t<T, D, true, true>(a, stages, st) : launch_bwd_t<T, D, true, false>(a, stages, st);
-  return drop ? launch_bwd_t<T, D, false, true>(a, stages, st) : launch_bwd_t<T, D, false, false>(a, stages, st);
+  if (drop) return launch_bwd_t<T, D, false, true>(a, stages, st);
+#endif
+  return launch_bwd_t<T, D, false, false>(a, stages, st);
 }
 
 hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t st) {
+#ifdef ACCT_DEV_BUILD
+  return launch_bwd_d<f16, 128>(a, stages, st);
+#else
   if (dtype == 0) {
     if (D == 128) return launch_bwd_d<f16, 128>(a, stages, st);
     if (D == 64) return launch_bwd_d<f16, 64>(a, stages, st);
@@ -513,6 +538,7 @@ hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t
     if (D == 80) return launch_bwd_d<bf16, 80>(a, stages, st);
   }
   return hipErrorInvalidValue;
+#endif
 }
 
 }  // namespace acct

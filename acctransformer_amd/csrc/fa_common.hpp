@@ -132,7 +132,7 @@ ACCT_DEV void load_bias4(const T* row, int kv, int limit, bool vec_ok, float out
 }
 
 // ---- 64-row tiles staged through LDS ---------------------------------------
-template <int D> struct TileCfg {
+template <int D, int NT = 256> struct TileCfg {
   static constexpr int KS = D / 16;             // 16-wide k-steps across the head dim
   static constexpr int DB = (D + 31) / 32;      // 32-wide blocks across the head dim
   static constexpr int DP = DB * 32;
@@ -140,15 +140,15 @@ template <int D> struct TileCfg {
   static constexpr int ROWB = DP * 2 + 16;      // LDS row pitch (bytes): +16 keeps b128 reads conflict free
   static constexpr int BN = 64;                 // rows per staged tile
   static constexpr int TILEB = BN * ROWB;
-  static constexpr int NLD = (BN * CPR + 255) / 256;
+  static constexpr int NLD = (BN * CPR + NT - 1) / NT;   // 16-byte chunks per thread and tile
 };
 
-template <typename T, int D>
-ACCT_DEV void tile_load(const T* base, int64_t row_stride, int row0, int nrows, u32x4 (&reg)[TileCfg<D>::NLD]) {
-  using C = TileCfg<D>;
+template <typename T, int D, int NT = 256>
+ACCT_DEV void tile_load(const T* base, int64_t row_stride, int row0, int nrows, u32x4 (&reg)[TileCfg<D, NT>::NLD]) {
+  using C = TileCfg<D, NT>;
 #pragma unroll
   for (int i = 0; i < C::NLD; i++) {
-    const int idx = threadIdx.x + 256 * i;
+    const int idx = threadIdx.x + NT * i;
     const int row = idx / C::CPR, ch = idx % C::CPR;
     u32x4 v = {0u, 0u, 0u, 0u};
     if (idx < C::BN * C::CPR && row0 + row < nrows)
@@ -157,15 +157,64 @@ ACCT_DEV void tile_load(const T* base, int64_t row_stride, int row0, int nrows, 
   }
 }
 
-template <int D>
-ACCT_DEV void tile_store(ACCT_LDS char* buf, const u32x4 (&reg)[TileCfg<D>::NLD]) {
-  using C = TileCfg<D>;
+template <int D, int NT = 256>
+ACCT_DEV void tile_store(ACCT_LDS char* buf, const u32x4 (&reg)[TileCfg<D, NT>::NLD]) {
+  using C = TileCfg<D, NT>;
 #pragma unroll
   for (int i = 0; i < C::NLD; i++) {
-    const int idx = threadIdx.x + 256 * i;
+    const int idx = threadIdx.x + NT * i;
     const int row = idx / C::CPR, ch = idx % C::CPR;
     if (idx < C::BN * C::CPR) *reinterpret_cast<ACCT_LDS u32x4*>(buf + row * C::ROWB + ch * 16) = reg[i];
   }
 }
+
+// ---- swizzled LDS tiles filled by direct-to-LDS loads --------------------------
+// Row pitch is a power of two (no padding, as the DMA writes 64 consecutive 16-byte
+// slots per wave instruction); the 16-byte chunk c of row r lives in slot c ^ (r & 7).
+// Eight consecutive rows then put one logical chunk into eight different 4-bank
+// groups, so both the 16-byte fragment reads (lane = row) and the transposed
+// 8-byte reads are free of bank conflicts.
+#define ACCT_GLB __attribute__((address_space(1)))
+
+template <int D> struct SwzCfg {
+  static constexpr int KS = D / 16;             // 16-wide k-steps across the head dim
+  static constexpr int DB = (D + 31) / 32;      // 32-wide blocks across the head dim
+  static constexpr int CPR = D / 8;             // valid 16-byte chunks per row
+  static constexpr int CH = D <= 64 ? 8 : 16;   // chunk slots per LDS row
+  static constexpr int PITCH = CH * 16;
+  static constexpr int RPI = 64 / CH;           // rows covered by one wave-wide DMA instruction
+};
+
+// Stage rows [row0, row0 + ROWS) of a row-major global matrix into a swizzled LDS
+// tile with NW waves.  Rows past nrows repeat the last valid row (finite data whose
+// contribution is zeroed by the caller's masking), slots past the valid chunks
+// repeat the last valid chunk.
+template <typename T, int D, int ROWS, int NW>
+ACCT_DEV void tile_dma(const T* base, int64_t row_stride, int row0, int nrows, ACCT_LDS char* buf) {
+  using C = SwzCfg<D>;
+  constexpr int NI = ROWS / C::RPI;
+  static_assert(NI % NW == 0, "tile rows must split evenly over the waves");
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < NI / NW; i++) {
+    const int inst = wave * (NI / NW) + i;
+    const int r = inst * C::RPI + lane / C::CH;
+    const int lc = min((lane % C::CH) ^ (r & 7), C::CPR - 1);
+    const int grow = min(row0 + r, nrows - 1);
+    const T* src = base + (int64_t)grow * row_stride + lc * 8;
+    // Issued as inline assembly on purpose: the compiler then does not order every later LDS read
+    // behind these loads (it cannot tell the two tile buffers apart), which would serialise the
+    // prefetch of the next tile with the work on the current one.  dma_wait() + the workgroup
+    // barrier publish the tile.
+    const uint32_t dst = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(buf + inst * 1024));
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(dst) : "memory");
+  }
+}
+
+// all of this wave's direct-to-LDS loads have landed
+ACCT_DEV void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// byte offset of logical chunk `lc` in a row whose (row & 7) is `swz`
+ACCT_DEV int swz_off(int lc, int swz) { return (lc ^ swz) << 4; }
 
 }  // namespace acct

@@ -18,14 +18,15 @@
 
 namespace acct {
 
-template <typename T, int D, int QG, bool BIAS, bool DROP>
-__global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
+template <typename T, int D, int QG, int NW, bool BIAS, bool DROP>
+__global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   using E = Elem<T>;
   using V8 = typename E::V8;
-  using C = TileCfg<D>;
-  constexpr int BM = 128 * QG;
+  using C = SwzCfg<D>;
+  constexpr int BM = 32 * QG * NW;
+  constexpr int TILEB = 64 * C::PITCH;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 buffers][K tile | V tile]
+  ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 buffers][K tile | V tile]; reused by the epilogue
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, g = lane >> 5;
   const int BH = a.B * a.N;
@@ -41,7 +42,7 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
   const T* kp = (const T*)a.k + b * a.k_sb + h * a.k_sh;
   const T* vp = (const T*)a.v + b * a.v_sb + h * a.v_sh;
 
-  // ---- visible kv tiles of this block (128-block band; causal clips the top) ----
+  // ---- visible kv tiles of this block (128-block band; causal and row-prefix clip the top) ----
   const int qb_lo = q0 / 128, qb_hi = (q_end - 1) / 128;
   const int kvb_lo = max(0, qb_lo - a.prev_blk), kvb_hi = min(a.Tc - 1, qb_hi + a.next_blk);
   int j_lo = kvb_lo * 2, j_hi = min(kvb_hi * 2 + 1, (a.Sk - 1) / 64);
@@ -55,13 +56,21 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
   V8 qf[QG][C::KS];
 #pragma unroll
   for (int gq = 0; gq < QG; gq++) {
-    const int row = wq0 + 32 * gq + l32;
+    const int row = min(wq0 + 32 * gq + l32, a.Sq - 1);     // rows past Sq repeat the last row; never stored
 #pragma unroll
-    for (int t = 0; t < C::KS; t++) {
-      V8 z = {};
-      qf[gq][t] = (row < a.Sq) ? *reinterpret_cast<const V8*>(qp + (int64_t)row * a.q_ss + 16 * t + 8 * g) : z;
-    }
+    for (int t = 0; t < C::KS; t++)
+      qf[gq][t] = *reinterpret_cast<const V8*>(qp + (int64_t)row * a.q_ss + 16 * t + 8 * g);
   }
+
+  // ---- per-lane LDS offsets (tile-invariant) ----
+  int koff[C::KS];                                          // K fragment of k-step t: row l32, chunk 2t + g
+#pragma unroll
+  for (int t = 0; t < C::KS; t++) koff[t] = l32 * C::PITCH + swz_off(2 * t + g, l32 & 7);
+  const int trow = 4 * g + ((lane & 15) >> 2);              // transposed reads: row within an 8-row group
+  const int tchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+  int voff[C::DB];                                          // V^T fragment of d block db
+#pragma unroll
+  for (int db = 0; db < C::DB; db++) voff[db] = trow * C::PITCH + swz_off(4 * db + tchunk, trow) + 8 * (lane & 1);
 
   f32x16 o[QG][C::DB];
   float m[QG], lsum[QG];
@@ -89,21 +98,18 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
   const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
   if (j_lo <= j_hi) {
-    u32x4 kreg[C::NLD], vreg[C::NLD];
-    tile_load<T, D>(kp, a.k_ss, j_lo * 64, a.Sk, kreg);
-    tile_load<T, D>(vp, a.v_ss, j_lo * 64, a.Sk, vreg);
-    tile_store<D>(smem, kreg);
-    tile_store<D>(smem + C::TILEB, vreg);
+    tile_dma<T, D, 64, NW>(kp, a.k_ss, j_lo * 64, a.Sk, smem);
+    tile_dma<T, D, 64, NW>(vp, a.v_ss, j_lo * 64, a.Sk, smem + TILEB);
+    dma_wait();
     __syncthreads();
 
     for (int j = j_lo; j <= j_hi; j++) {
       const int buf = (j - j_lo) & 1;
-      ACCT_LDS char* kbuf = smem + buf * 2 * C::TILEB;
-      ACCT_LDS char* vbuf = kbuf + C::TILEB;
-      const bool more = j < j_hi;
-      if (more) {
-        tile_load<T, D>(kp, a.k_ss, (j + 1) * 64, a.Sk, kreg);
-        tile_load<T, D>(vp, a.v_ss, (j + 1) * 64, a.Sk, vreg);
+      ACCT_LDS char* kbuf = smem + buf * 2 * TILEB;
+      ACCT_LDS char* vbuf = kbuf + TILEB;
+      if (j < j_hi) {                                       // next tile streams into the other buffer meanwhile
+        tile_dma<T, D, 64, NW>(kp, a.k_ss, (j + 1) * 64, a.Sk, smem + (buf ^ 1) * 2 * TILEB);
+        tile_dma<T, D, 64, NW>(vp, a.v_ss, (j + 1) * 64, a.Sk, smem + (buf ^ 1) * 2 * TILEB + TILEB);
       }
       const int kv0 = j * 64;
       const int kvb = j >> 1;
@@ -127,18 +133,21 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
           for (int c = 0; c < 2; c++)
 #pragma unroll
             for (int r = 0; r < 16; r++) s[gq][c][r] = 0.f;
+        {
+          V8 kf[2][C::KS];                                  // every K fragment of the tile is requested up front;
+#pragma unroll                                              // the MFMAs then start as the reads return in order
+          for (int c = 0; c < 2; c++)
 #pragma unroll
-        for (int t = 0; t < C::KS; t++) {
+            for (int t = 0; t < C::KS; t++) kf[c][t] = lds_read_frag<T>(kbuf + koff[t] + c * 32 * C::PITCH);
 #pragma unroll
-          for (int c = 0; c < 2; c++) {
-            const V8 kf = lds_read_frag<T>(kbuf + (32 * c + l32) * C::ROWB + (16 * t + 8 * g) * 2);
+          for (int c = 0; c < 2; c++)
 #pragma unroll
-            for (int gq = 0; gq < QG; gq++) s[gq][c] = E::mfma(kf, qf[gq][t], s[gq][c]);
-          }
+            for (int t = 0; t < C::KS; t++)
+#pragma unroll
+              for (int gq = 0; gq < QG; gq++) s[gq][c] = E::mfma(kf[c][t], qf[gq][t], s[gq][c]);
         }
         // element (gq, c, r): q = wq0 + 32 gq + l32 ; kv = kv0 + 32 c + 8 (r/4) + 4 g + r%4
-        const bool tail = kv0 + 64 > a.Sk;
-        const bool diag = causal && (kv0 + 63 > wq0);
+        const bool edge = apply_mask || (causal && (kv0 + 63 > wq0)) || (kv0 + 64 > a.Sk);
         typename E::V8 pf[QG][2][2];
 #pragma unroll
         for (int gq = 0; gq < QG; gq++) {
@@ -157,7 +166,7 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
                   s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale_log2e, bias[e] * kLog2e);
               }
           }
-          if (apply_mask || diag || tail) {
+          if (edge) {
 #pragma unroll
             for (int c = 0; c < 2; c++)
 #pragma unroll
@@ -234,75 +243,90 @@ __global__ void __launch_bounds__(256) fa_fwd_kernel(const FaArgs a) {
           for (int hh = 0; hh < 2; hh++)
 #pragma unroll
             for (int db = 0; db < C::DB; db++) {
-              const ACCT_LDS char* vaddr = vbuf + (32 * c + 16 * hh + 4 * g + ((lane & 15) >> 2)) * C::ROWB +
-                                           (32 * db + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
-              const V8 vf = join_tr<T>(lds_read_tr(vaddr), lds_read_tr(vaddr + 8 * C::ROWB));
+              const ACCT_LDS char* vaddr = vbuf + voff[db] + (32 * c + 16 * hh) * C::PITCH;
+              const V8 vf = join_tr<T>(lds_read_tr(vaddr), lds_read_tr(vaddr + 8 * C::PITCH));
 #pragma unroll
               for (int gq = 0; gq < QG; gq++) o[gq][db] = E::mfma(vf, pf[gq][c][hh], o[gq][db]);
             }
       }
-      if (more) {
-        ACCT_LDS char* nk = smem + (buf ^ 1) * 2 * C::TILEB;
-        tile_store<D>(nk, kreg);
-        tile_store<D>(nk + C::TILEB, vreg);
-      }
+      dma_wait();
       __syncthreads();
     }
   }
 
-  // ---- epilogue: O = O^T / l, LSE = m + ln l ----
+  // ---- epilogue: O = O^T / l, LSE = m + ln l.  Each wave transposes its rows through its own
+  // LDS region (pitch 2D+16 keeps the 8-byte writes of 16 rows on distinct banks) so that the
+  // global stores are whole rows. ----
   T* op = (T*)a.o + b * a.o_sb + h * a.o_sh;
   const float mnat = BIAS ? kLn2 : a.scale;
+  constexpr int OPITCH = C::DB * 64 + 16;
+  ACCT_LDS char* obuf = smem + wave * (32 * OPITCH);
 #pragma unroll
   for (int gq = 0; gq < QG; gq++) {
     const int row = wq0 + 32 * gq + l32;
     const float l = pair_sum(lsum[gq]);
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    if (row < a.Sq) {
-      if (g == 0) a.lse[(int64_t)bh * a.Sq + row] = l > 0.f ? m[gq] * mnat + __logf(l) : -INFINITY;
+    if (row < a.Sq && g == 0) a.lse[(int64_t)bh * a.Sq + row] = l > 0.f ? m[gq] * mnat + __logf(l) : -INFINITY;
 #pragma unroll
-      for (int db = 0; db < C::DB; db++)
+    for (int db = 0; db < C::DB; db++)
 #pragma unroll
-        for (int r4 = 0; r4 < 4; r4++) {
-          const int d = 32 * db + 8 * r4 + 4 * g;
-          if (d < D) {
-            typename E::V2 t0 = E::cvt2(o[gq][db][4 * r4 + 0] * inv, o[gq][db][4 * r4 + 1] * inv);
-            typename E::V2 t1 = E::cvt2(o[gq][db][4 * r4 + 2] * inv, o[gq][db][4 * r4 + 3] * inv);
-            typename E::V4 ov = {t0[0], t0[1], t1[0], t1[1]};
-            *reinterpret_cast<typename E::V4*>(op + (int64_t)row * a.o_ss + d) = ov;
-          }
-        }
+      for (int r4 = 0; r4 < 4; r4++) {
+        typename E::V2 t0 = E::cvt2(o[gq][db][4 * r4 + 0] * inv, o[gq][db][4 * r4 + 1] * inv);
+        typename E::V2 t1 = E::cvt2(o[gq][db][4 * r4 + 2] * inv, o[gq][db][4 * r4 + 3] * inv);
+        typename E::V4 ov = {t0[0], t0[1], t1[0], t1[1]};
+        *reinterpret_cast<ACCT_LDS typename E::V4*>(obuf + l32 * OPITCH + (32 * db + 8 * r4 + 4 * g) * 2) = ov;
+      }
+    // read back row-contiguous: 16-byte chunk ch of row r
+    constexpr int NCH = C::CPR;                      // valid chunks per row
+#pragma unroll
+    for (int i = 0; i < (32 * NCH + 63) / 64; i++) {
+      const int idx = lane + 64 * i;
+      const int r = idx / NCH, ch = idx % NCH;
+      const int grow = wq0 + 32 * gq + r;
+      if (idx < 32 * NCH && grow < a.Sq) {
+        const u32x4 v = *reinterpret_cast<const ACCT_LDS u32x4*>(obuf + r * OPITCH + ch * 16);
+        *reinterpret_cast<u32x4*>(op + (int64_t)grow * a.o_ss + ch * 8) = v;
+      }
     }
   }
 }
 
-template <typename T, int D, int QG, bool BIAS, bool DROP>
+template <typename T, int D, int QG, int NW, bool BIAS, bool DROP>
 static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
-  using C = TileCfg<D>;
-  constexpr int BM = 128 * QG;
+  using C = SwzCfg<D>;
+  constexpr int BM = 32 * QG * NW;
   a.n_tiles = (a.Sq + BM - 1) / BM;
-  const size_t smem = 4 * (size_t)C::TILEB;
-  auto kern = fa_fwd_kernel<T, D, QG, BIAS, DROP>;
+  constexpr size_t tiles = 4 * 64 * (size_t)C::PITCH, stage = (size_t)NW * 32 * (C::DB * 64 + 16);
+  const size_t smem = tiles > stage ? tiles : stage;
+  auto kern = fa_fwd_kernel<T, D, QG, NW, BIAS, DROP>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (e != hipSuccess) return e;
   const long long nblk = (long long)a.n_tiles * a.B * a.N;
-  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(256), smem, st, a);
+  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(64 * NW), smem, st, a);
   return hipGetLastError();
 }
 
-template <typename T, int D, int QG>
+template <typename T, int D, int QG, int NW>
 static hipError_t launch_fwd_q(const FaArgs& a, hipStream_t st) {
   const bool bias = a.alibi != nullptr, drop = a.drop != nullptr;
-  if (bias) return drop ? launch_fwd_t<T, D, QG, true, true>(a, st) : launch_fwd_t<T, D, QG, true, false>(a, st);
-  return drop ? launch_fwd_t<T, D, QG, false, true>(a, st) : launch_fwd_t<T, D, QG, false, false>(a, st);
+#ifndef ACCT_DEV_BUILD
+  if (bias) return drop ? launch_fwd_t<T, D, QG, NW, true, true>(a, st) : launch_fwd_t<T, D, QG, NW, true, false>(a, st);
+  if (drop) return launch_fwd_t<T, D, QG, NW, false, true>(a, st);
+#endif
+  return launch_fwd_t<T, D, QG, NW, false, false>(a, st);
 }
 
+// variant: 1 = 4 waves x 32 rows, 2 = 4 waves x 64 rows, 3 = 8 waves x 32 rows
 template <typename T, int D>
-static hipError_t launch_fwd_d(const FaArgs& a, int qg, hipStream_t st) {
-  return qg == 2 ? launch_fwd_q<T, D, 2>(a, st) : launch_fwd_q<T, D, 1>(a, st);
+static hipError_t launch_fwd_d(const FaArgs& a, int variant, hipStream_t st) {
+  if (variant == 3) return launch_fwd_q<T, D, 1, 8>(a, st);
+  return variant == 2 ? launch_fwd_q<T, D, 2, 4>(a, st) : launch_fwd_q<T, D, 1, 4>(a, st);
 }
 
 hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st) {
+#ifdef ACCT_DEV_BUILD
+  return launch_fwd_d<f16, 128>(a, qg, st);
+#else
   if (dtype == 0) {
     if (D == 128) return launch_fwd_d<f16, 128>(a, qg, st);
     if (D == 64) return launch_fwd_d<f16, 64>(a, qg, st);
@@ -313,6 +337,7 @@ hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st)
     if (D == 80) return launch_fwd_d<bf16, 80>(a, qg, st);
   }
   return hipErrorInvalidValue;
+#endif
 }
 
 }  // namespace acct
