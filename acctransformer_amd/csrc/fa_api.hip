@@ -109,6 +109,7 @@ acct::FaArgs make_args(const acct_fa_params* p) {
   a.scale = p->scale;
   a.scale_log2e = p->scale * acct::kLog2e;
   a.inv_keep = 1.0f / p->keep_prob;
+  a.inv_scale = 1.0f / p->scale;
   a.mask_add_raw = acct::kMaskFill / p->scale;
   a.prev_blk = p->prev_block_num > ACCT_BLOCK_UNBOUNDED ? ACCT_BLOCK_UNBOUNDED : p->prev_block_num;
   a.next_blk = p->next_block_num > ACCT_BLOCK_UNBOUNDED ? ACCT_BLOCK_UNBOUNDED : p->next_block_num;

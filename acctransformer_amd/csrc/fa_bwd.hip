@@ -270,25 +270,47 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 }
 
 // ============================================================================
-// dK/dV kernel: kv-tile owner.  Each wave owns 32*KG key rows; Q and dO tiles of
-// 64 query rows are staged through LDS.
+// dK/dV kernel: kv-tile owner, 8 waves in 4 pairs.  A pair owns 64 key rows.
+// Its first wave (V role) keeps the K fragments of those rows in registers,
+// recomputes S = Q K^T and P, hands P (fp16) to its partner through LDS and
+// accumulates dV^T += dO^T P.  The partner (K role) keeps the V fragments,
+// computes dP = dO V^T, forms dS = P*(dP - D) and accumulates dK^T += Q^T dS.
+// Splitting the two accumulators over two waves halves the registers per wave
+// (two waves fit on each SIMD and overlap each other's MFMA and exp/convert
+// phases) while every Q / dO fragment read from LDS still feeds two MFMAs.
 // ============================================================================
-template <typename T, int D, int KG, bool BIAS, bool DROP>
-__global__ void __launch_bounds__(256) fa_bwd_dkdv_kernel(const FaArgs a) {
+#ifndef ACCT_PARK
+#define ACCT_PARK 6
+#endif
+ACCT_DEV void dma4(const void* src, ACCT_LDS char* dst) {
+  const uint32_t d = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(d) : "memory");
+}
+
+template <typename T, int D, bool BIAS, bool DROP>
+__global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   using E = Elem<T>;
   using V8 = typename E::V8;
-  using C = TileCfg<D>;
-  constexpr int BNK = 128 * KG;                     // key rows per workgroup
+  using C = SwzCfg<D>;
+  constexpr int NW = 8;
+  constexpr int BNK = 256;                          // key rows per workgroup
+  constexpr int TILEB = 64 * C::PITCH;
+  constexpr int STATB = 2 * 64 * 4;                 // LSE and D of the 64 rows of a tile
+  constexpr int STAGEB = 2 * TILEB + STATB;         // one buffer: Q tile | dO tile | LSE | D
+  constexpr int PXB = 4096;                         // P of one pair and chunk: 64 lanes x 64 bytes
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 buffers][Q tile | dO tile]
+  ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 stage buffers][2 x 4 pair P buffers]
+  ACCT_LDS char* pexch = smem + 2 * STAGEB;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, g = lane >> 5;
+  const int pair = wave & 3;
+  const bool krole = wave >= 4;                     // false: V role (S, P, dV); true: K role (dP, dS, dK)
   const int BH = a.B * a.N;
   const int bh = blockIdx.x % BH;
   const int kt = (int)(blockIdx.x / BH);            // causal: the first key tiles are the heaviest
   const int b = bh / a.N, h = bh % a.N;
   const int k0 = kt * BNK;
-  const int wk0 = k0 + wave * 32 * KG;              // first key row of this wave
+  const int wk0 = k0 + pair * 64;                   // first key row of this pair
   const int k_end = min(k0 + BNK, a.Sk);
 
   const T* qp = (const T*)a.q + b * a.q_sb + h * a.q_sh;
@@ -306,187 +328,270 @@ __global__ void __launch_bounds__(256) fa_bwd_dkdv_kernel(const FaArgs a) {
   if (causal) i_lo = max(i_lo, k0 / 64);            // query tiles wholly above the diagonal contribute 0
   const int wkb = wk0 / 128;
 
-  // K and V fragments of the wave's key rows (B operands): lane holds key row l32, d = 16t + 8g ..
-  V8 kf[KG][C::KS], vf[KG][C::KS];
+  // stationary B operands: K fragments (V role) or V fragments (K role) of the pair's 64 key rows;
+  // lane holds key row 32 gk + l32, d = 16t + 8g ..
+  // The last PARK k-steps of the second key group live in a wave-private LDS slab instead of
+  // registers (16 VGPRs at D = 128): that is what lets two waves share a SIMD without spilling.
+  constexpr int PARK = D >= 128 ? ACCT_PARK : 0;
+  V8 bf[2][C::KS];
+  ACCT_LDS char* park = pexch + 8 * PXB + wave * (PARK * 1024) + lane * 16;
+  {
+    const T* src = krole ? vp : kp;
+    const int64_t ss = krole ? a.v_ss : a.k_ss;
 #pragma unroll
-  for (int gk = 0; gk < KG; gk++) {
-    const int row = wk0 + 32 * gk + l32;
+    for (int gk = 0; gk < 2; gk++) {
+      const int row = min(wk0 + 32 * gk + l32, a.Sk - 1);
 #pragma unroll
-    for (int t = 0; t < C::KS; t++) {
-      V8 z = {};
-      kf[gk][t] = z;
-      vf[gk][t] = z;
-      if (row < a.Sk) {
-        kf[gk][t] = *reinterpret_cast<const V8*>(kp + (int64_t)row * a.k_ss + 16 * t + 8 * g);
-        vf[gk][t] = *reinterpret_cast<const V8*>(vp + (int64_t)row * a.v_ss + 16 * t + 8 * g);
+      for (int t = 0; t < C::KS; t++) {
+        const V8 v = *reinterpret_cast<const V8*>(src + (int64_t)row * ss + 16 * t + 8 * g);
+        if (gk == 1 && t >= C::KS - PARK) *reinterpret_cast<ACCT_LDS V8*>(park + (t - (C::KS - PARK)) * 1024) = v;
+        else bf[gk][t] = v;
       }
     }
   }
-  f32x16 dk[KG][C::DB], dv[KG][C::DB];
+  f32x16 acc[2][C::DB];                             // dV^T (V role) or dK^T (K role): [d rows, key column l32]
 #pragma unroll
-  for (int gk = 0; gk < KG; gk++)
+  for (int gk = 0; gk < 2; gk++)
 #pragma unroll
     for (int db = 0; db < C::DB; db++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) { dk[gk][db][r] = 0.f; dv[gk][db][r] = 0.f; }
+      for (int r = 0; r < 16; r++) acc[gk][db][r] = 0.f;
+
+  // per-lane LDS offsets (tile-invariant)
+#define FOFF(t) (foff4[(t) & 3] + ((t) >> 2) * 128)
+#define TOFF(db) (toff2[(db) & 1] + ((db) >> 1) * 128)
+#ifdef ACCT_NO_EDGE
+#define EDGE_PATH false
+#else
+#define EDGE_PATH edge
+#endif
 
   const int mb = a.mask_sb ? b : 0;
   const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
   const uint8_t* dropp = DROP ? a.drop + ((int64_t)bh * a.Sq) * a.Sk : nullptr;
   const T* alibip = BIAS ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
-  const bool stat_vec = ((((uintptr_t)lsep | (uintptr_t)delp) & 15) == 0);
+
+  // stage q tile i into buffer `sb`: Q and dO by 16-byte DMA (2 instructions per wave each),
+  // LSE (wave 0) and D (wave 1) by 4-byte DMA; rows past Sq repeat the last row
+  auto stage = [&](int i, ACCT_LDS char* sb) {
+    tile_dma<T, D, 64, NW>(qp, a.q_ss, i * 64, a.Sq, sb);
+    tile_dma<T, D, 64, NW>(dop, a.o_ss, i * 64, a.Sq, sb + TILEB);
+    if (wave < 2) {
+      const int r = min(i * 64 + lane, a.Sq - 1);
+      dma4((wave == 0 ? lsep : delp) + r, sb + 2 * TILEB + wave * 256);
+    }
+  };
+
+  // per-chunk predicates of this pair (chunk = 32 query rows; two per staged tile)
+  auto classify = [&](int cidx, bool& act, bool& apply_mask, bool& edge) {
+    const int qc0 = cidx * 32, qt0 = (cidx >> 1) * 64, qb = cidx >> 2;
+    act = (wkb - a.next_blk <= qb) && (qb <= wkb + a.prev_blk) && (wk0 < a.Sk);
+    if (causal) act = act && (qt0 + 63 >= wk0);
+    if (a.row_prefix) act = act && (wk0 < (qt0 / a.row_prefix + 1) * a.row_prefix);
+    apply_mask = false;
+    if (a.mask_kind == kMaskDense && act) {
+      const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + qb) * a.Tc + wkb];
+      act = f != kBlkSkip;
+      apply_mask = f == kBlkApply;
+    } else if (a.mask_kind == kMaskTile) {
+      apply_mask = wkb == qb;
+    }
+    edge = BIAS || DROP || apply_mask || (causal && (wk0 + 63 > qc0)) || (wk0 + 64 > a.Sk) || (qc0 + 32 > a.Sq);
+  };
 
   if (i_lo <= i_hi) {
-    u32x4 qreg[C::NLD], doreg[C::NLD];
-    tile_load<T, D>(qp, a.q_ss, i_lo * 64, a.Sq, qreg);
-    tile_load<T, D>(dop, a.o_ss, i_lo * 64, a.Sq, doreg);
-    tile_store<D>(smem, qreg);
-    tile_store<D>(smem + C::TILEB, doreg);
+    stage(i_lo, smem);
+    dma_wait();
     __syncthreads();
 
-    for (int i = i_lo; i <= i_hi; i++) {
-      const int buf = (i - i_lo) & 1;
-      ACCT_LDS char* qbuf = smem + buf * 2 * C::TILEB;
-      ACCT_LDS char* dobuf = qbuf + C::TILEB;
-      const bool more = i < i_hi;
-      if (more) {
-        tile_load<T, D>(qp, a.q_ss, (i + 1) * 64, a.Sq, qreg);
-        tile_load<T, D>(dop, a.o_ss, (i + 1) * 64, a.Sq, doreg);
-      }
-      const int qt0 = i * 64;
-      const int qb = i >> 1;
-      bool act = (wkb - a.next_blk <= qb) && (qb <= wkb + a.prev_blk) && (wk0 < a.Sk);
-      if (causal) act = act && (qt0 + 63 >= wk0);
-      if (a.row_prefix) act = act && (wk0 < (qt0 / a.row_prefix + 1) * a.row_prefix);
-      bool apply_mask = false;
-      if (a.mask_kind == kMaskDense && act) {
-        const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + qb) * a.Tc + wkb];
-        act = f != kBlkSkip;
-        apply_mask = f == kBlkApply;
-      } else if (a.mask_kind == kMaskTile) {
-        apply_mask = wkb == qb;
-      }
-      const bool diag = causal && (wk0 + 32 * KG - 1 > qt0);
-      if (act) {
+    // The K role runs one chunk behind the V role: in step n the V role recomputes P of chunk n,
+    // publishes it and accumulates dV; the K role picks up P of chunk n-1.  One barrier per step,
+    // nothing is carried across it in registers.
+    const int c_lo = 2 * i_lo, c_hi = 2 * i_hi + 1;
+    for (int n = c_lo; n <= c_hi + 1; n++) {
+      if ((n & 1) && (n >> 1) < i_hi) stage((n >> 1) + 1, smem + ((((n >> 1) + 1 - i_lo) & 1) * STAGEB));
+      const int cidx = krole ? n - 1 : n;             // the chunk this wave works on in this step
+      if (cidx >= c_lo && cidx <= c_hi) {
+        bool act, apply_mask, edge;
+        classify(cidx, act, apply_mask, edge);
+        if (act) {
+          const int c = cidx & 1, qc0 = cidx * 32;
+          // Per-lane LDS offsets are re-derived in every step (a handful of VALU ops) rather than
+          // kept in registers.  The swizzle only touches the low three bits of the chunk index, so
+          // chunk c + 8 sits 128 bytes after chunk c: four (two) base offsets plus immediates cover
+          // all fragments of a row.
+          int ln = lane;
+          asm volatile("" : "+v"(ln));
+          int foff4[4];                               // row-major fragment of k-step t: row l32, chunk 2t + g
 #pragma unroll
-        for (int c = 0; c < 2; c++) {                 // 32-row query chunk of the tile
-          // rows of this lane's C registers: q = qt0 + 32 c + 8 (r/4) + 4 g + r%4
-          float lrow[16], drow[16];
+          for (int t = 0; t < 4; t++) foff4[t] = (ln & 31) * C::PITCH + swz_off(2 * t + (ln >> 5), ln & 7);
+          const int trow = 4 * (ln >> 5) + ((ln & 15) >> 2);
+          const int tchunk = 2 * ((ln >> 4) & 1) + ((ln & 3) >> 1);
+          int toff2[2];                               // transposed fragment of d block db
 #pragma unroll
-          for (int r4 = 0; r4 < 4; r4++) {
-            const int q = qt0 + 32 * c + 8 * r4 + 4 * g;
-            load_f32x4(lsep, q, a.Sq, stat_vec, INFINITY, lrow + 4 * r4);
-            load_f32x4(delp, q, a.Sq, stat_vec, 0.f, drow + 4 * r4);
-          }
-          f32x16 s[KG], dp[KG];
+          for (int db = 0; db < 2; db++) toff2[db] = trow * C::PITCH + swz_off(4 * db + tchunk, trow) + 8 * (ln & 1);
+          ACCT_LDS char* qbuf = smem + (((cidx >> 1) - i_lo) & 1) * STAGEB;
+          ACCT_LDS char* dobuf = qbuf + TILEB;
+          const ACCT_LDS float* lbuf = (const ACCT_LDS float*)(qbuf + 2 * TILEB);
+          const ACCT_LDS float* dbuf = lbuf + 64;
+          ACCT_LDS char* px = pexch + ((cidx & 1) * 4 + pair) * PXB + ln * 16;
+          // rows of this lane's C registers: q = qc0 + 8 (r/4) + 4 g + r%4 ; key = wk0 + 32 gk + l32
+          f32x16 t0[2];                               // S (V role) or dP (K role) of the two key groups
 #pragma unroll
-          for (int gk = 0; gk < KG; gk++)
+          for (int gk = 0; gk < 2; gk++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) { s[gk][r] = 0.f; dp[gk][r] = 0.f; }
+            for (int r = 0; r < 16; r++) t0[gk][r] = 0.f;
+          {
+            const ACCT_LDS char* abuf = (krole ? dobuf : qbuf) + c * 32 * C::PITCH;
 #pragma unroll
-          for (int t = 0; t < C::KS; t++) {
-            const V8 qa = lds_read_frag<T>(qbuf + (32 * c + l32) * C::ROWB + (16 * t + 8 * g) * 2);
-            const V8 doa = lds_read_frag<T>(dobuf + (32 * c + l32) * C::ROWB + (16 * t + 8 * g) * 2);
+            for (int t = 0; t < C::KS; t++) {
+              const V8 af = lds_read_frag<T>(abuf + FOFF(t));
 #pragma unroll
-            for (int gk = 0; gk < KG; gk++) {
-              s[gk] = E::mfma(qa, kf[gk][t], s[gk]);       // S[q, kv]
-              dp[gk] = E::mfma(doa, vf[gk][t], dp[gk]);    // dP[q, kv]
+              for (int gk = 0; gk < 2; gk++) {                                             // S[q, key] or dP[q, key]
+                const V8 b = (gk == 1 && t >= C::KS - PARK) ? *reinterpret_cast<const ACCT_LDS V8*>(park + (t - (C::KS - PARK)) * 1024)
+                                                            : bf[gk][t];
+                t0[gk] = E::mfma(af, b, t0[gk]);
+              }
             }
           }
-          V8 pf[KG][2], dsf[KG][2];
-#pragma unroll
-          for (int gk = 0; gk < KG; gk++) {
-            const int kv = wk0 + 32 * gk + l32;
-            const int kv_c = min(kv, a.Sk - 1);
-            float pv[16], ds[16];
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-              const int q = qt0 + 32 * c + 8 * (r >> 2) + 4 * g + (r & 3);
-              const int q_c = min(q, a.Sq - 1);
-              float x = __builtin_fmaf(s[gk][r], a.scale_log2e, -lrow[r] * kLog2e);
-              bool keep = true;
-              if (BIAS) x = __builtin_fmaf((float)alibip[(int64_t)q_c * a.al_sq + kv_c], kLog2e, x);
+          V8 bfr[2][2];                               // B fragments of the second product: P (V role) or dS (K role)
+          if (!krole) {
+            if (EDGE_PATH) {
+              // side inputs and range limits are folded into the raw scores in place: +bias/scale,
+              // -10000/scale where masked, -inf where the key or the query row does not exist.
+              // Uniform 64-bit row bases + 32-bit per-lane offsets keep this path light on registers.
+              const int qlast = a.Sq - 1 - qc0;                 // last valid row, relative to the chunk
+              const uint8_t* mrow0 = nullptr;
+              int mstride = 0;
               if (apply_mask) {
-                const uint8_t mbyte = a.mask_kind == kMaskDense ? maskp[(int64_t)q_c * a.Sk + kv_c]
-                                                                : maskp[(q_c & 127) * 128 + (kv_c & 127)];
-                if (mbyte) x += kMaskFill * kLog2e;
+                if (a.mask_kind == kMaskDense) { mrow0 = maskp + (int64_t)qc0 * a.Sk; mstride = a.Sk; }
+                else { mrow0 = maskp + (qc0 & 127) * 128; mstride = 128; }
               }
-              if (DROP) keep = dropp[(int64_t)q_c * a.Sk + kv_c] != 0;
-              if (diag && kv > q) x += kMaskFill * kLog2e;
-              float p = fast_exp2(x);
-              if (kv >= a.Sk) p = 0.f;
-              float dpv = dp[gk][r];
-              float pd = p;
-              if (DROP) {
-                dpv = keep ? dpv * a.inv_keep : 0.f;
-                pd = keep ? p * a.inv_keep : 0.f;
+              const T* brow0 = BIAS ? alibip + (int64_t)qc0 * a.al_sq : nullptr;
+#pragma unroll
+              for (int gk = 0; gk < 2; gk++) {
+                const int kv = wk0 + 32 * gk + l32;
+                const int kv_c = min(kv, a.Sk - 1);
+                const int mcol = a.mask_kind == kMaskDense ? kv_c : (kv_c & 127);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                  const int qr = 8 * (r >> 2) + 4 * g + (r & 3);   // row within the chunk
+                  const int qr_c = min(qr, qlast);
+                  float x = t0[gk][r];
+                  if (BIAS) x += (float)brow0[qr_c * (int)a.al_sq + kv_c] * a.inv_scale;
+                  if (apply_mask && mrow0[qr_c * mstride + mcol]) x += a.mask_add_raw;
+                  if (causal && kv > qc0 + qr) x += a.mask_add_raw;
+                  if (kv >= a.Sk || qr > qlast) x = -INFINITY;
+                  t0[gk][r] = x;
+                  if ((r & 3) == 3) asm volatile("" ::: "memory");   // keep the side-input loads in small batches
+                }
               }
-              pv[r] = pd;
-              ds[r] = p * (dpv - drow[r]);
             }
-            pf[gk][0] = pack8<T>(pv);
-            pf[gk][1] = pack8<T>(pv + 8);
-            dsf[gk][0] = pack8<T>(ds);
-            dsf[gk][1] = pack8<T>(ds + 8);
+#pragma unroll
+            for (int gk = 0; gk < 2; gk++) {
+              const int kv_c = min(wk0 + 32 * gk + l32, a.Sk - 1);
+#pragma unroll
+              for (int hh = 0; hh < 2; hh++) {
+                float p[8], pd[8];
+#pragma unroll
+                for (int r4 = 0; r4 < 2; r4++) {
+                  const f32x4 lv = *reinterpret_cast<const ACCT_LDS f32x4*>(lbuf + 32 * c + 16 * hh + 8 * r4 + 4 * g);
+#pragma unroll
+                  for (int e = 0; e < 4; e++) {
+                    p[4 * r4 + e] = fast_exp2(__builtin_fmaf(t0[gk][8 * hh + 4 * r4 + e], a.scale_log2e, lv[e] * -kLog2e));
+                    pd[4 * r4 + e] = p[4 * r4 + e];
+                    if (DROP) {
+                      const int q_c = min(qc0 + 16 * hh + 8 * r4 + 4 * g + e, a.Sq - 1);
+                      pd[4 * r4 + e] = dropp[(int64_t)q_c * a.Sk + kv_c] ? p[4 * r4 + e] * a.inv_keep : 0.f;
+                    }
+                  }
+                }
+                bfr[gk][hh] = pack8<T>(pd);
+                // un-dropped P for the partner, always fp16 (P <= 1: finer than bf16)
+                *reinterpret_cast<ACCT_LDS f16x8*>(px + (2 * gk + hh) * 1024) = pack8<f16>(p);
+              }
+            }
+          } else {
+#pragma unroll
+            for (int gk = 0; gk < 2; gk++) {
+              const int kv_c = min(wk0 + 32 * gk + l32, a.Sk - 1);
+#pragma unroll
+              for (int hh = 0; hh < 2; hh++) {
+                const f16x8 ph = *reinterpret_cast<const ACCT_LDS f16x8*>(px + (2 * gk + hh) * 1024);
+                float ds[8];
+#pragma unroll
+                for (int r4 = 0; r4 < 2; r4++) {
+                  const f32x4 dv4 = *reinterpret_cast<const ACCT_LDS f32x4*>(dbuf + 32 * c + 16 * hh + 8 * r4 + 4 * g);
+#pragma unroll
+                  for (int e = 0; e < 4; e++) {
+                    float dpv = t0[gk][8 * hh + 4 * r4 + e];
+                    if (DROP) {
+                      const int q_c = min(qc0 + 16 * hh + 8 * r4 + 4 * g + e, a.Sq - 1);
+                      dpv = dropp[(int64_t)q_c * a.Sk + kv_c] ? dpv * a.inv_keep : 0.f;
+                    }
+                    ds[4 * r4 + e] = (float)ph[4 * r4 + e] * (dpv - dv4[e]);
+                  }
+                }
+                bfr[gk][hh] = pack8<T>(ds);
+              }
+            }
           }
-          // ---- dV^T += dO^T P ; dK^T += Q^T dS  (contract over the 32 query rows of chunk c) ----
+          // dV^T += dO^T P (V role) ; dK^T += Q^T dS (K role): contract over the 32 query rows of the chunk
+          const ACCT_LDS char* tb = (krole ? qbuf : dobuf) + c * 32 * C::PITCH;
 #pragma unroll
           for (int hh = 0; hh < 2; hh++)
 #pragma unroll
             for (int db = 0; db < C::DB; db++) {
-              const int off = (32 * c + 16 * hh + 4 * g + ((lane & 15) >> 2)) * C::ROWB +
-                              (32 * db + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
-              const V8 dot = join_tr<T>(lds_read_tr(dobuf + off), lds_read_tr(dobuf + off + 8 * C::ROWB));
-              const V8 qtf = join_tr<T>(lds_read_tr(qbuf + off), lds_read_tr(qbuf + off + 8 * C::ROWB));
+              const ACCT_LDS char* ta = tb + TOFF(db) + 16 * hh * C::PITCH;
+              const V8 af = join_tr<T>(lds_read_tr(ta), lds_read_tr(ta + 8 * C::PITCH));
 #pragma unroll
-              for (int gk = 0; gk < KG; gk++) {
-                dv[gk][db] = E::mfma(dot, pf[gk][hh], dv[gk][db]);
-                dk[gk][db] = E::mfma(qtf, dsf[gk][hh], dk[gk][db]);
-              }
+              for (int gk = 0; gk < 2; gk++) acc[gk][db] = E::mfma(af, bfr[gk][hh], acc[gk][db]);
             }
         }
       }
-      if (more) {
-        ACCT_LDS char* nq = smem + (buf ^ 1) * 2 * C::TILEB;
-        tile_store<D>(nq, qreg);
-        tile_store<D>(nq + C::TILEB, doreg);
-      }
+      dma_wait();                                     // a tile requested at the top of this step has landed
       __syncthreads();
     }
   }
 
-  // ---- epilogue ----
-  T* dkp = (T*)a.dk + b * a.k_sb + h * a.k_sh;
-  T* dvp = (T*)a.dv + b * a.v_sb + h * a.v_sh;
+  // ---- epilogue: dV (V role) / scale * dK (K role), transposed through the wave's own LDS region ----
+  T* outp = krole ? (T*)a.dk + b * a.k_sb + h * a.k_sh : (T*)a.dv + b * a.v_sb + h * a.v_sh;
+  const int64_t oss = krole ? a.k_ss : a.v_ss;
+  const float oscale = krole ? a.scale : 1.0f;
+  constexpr int OPITCH = C::DB * 64 + 16;
+  ACCT_LDS char* obuf = smem + wave * (32 * OPITCH);
 #pragma unroll
-  for (int gk = 0; gk < KG; gk++) {
-    const int row = wk0 + 32 * gk + l32;
-    if (row < a.Sk) {
+  for (int gk = 0; gk < 2; gk++) {
 #pragma unroll
-      for (int db = 0; db < C::DB; db++)
+    for (int db = 0; db < C::DB; db++)
 #pragma unroll
-        for (int r4 = 0; r4 < 4; r4++) {
-          const int d = 32 * db + 8 * r4 + 4 * g;
-          if (d < D) {
-            typename E::V2 t0 = E::cvt2(dk[gk][db][4 * r4 + 0] * a.scale, dk[gk][db][4 * r4 + 1] * a.scale);
-            typename E::V2 t1 = E::cvt2(dk[gk][db][4 * r4 + 2] * a.scale, dk[gk][db][4 * r4 + 3] * a.scale);
-            typename E::V4 kvv = {t0[0], t0[1], t1[0], t1[1]};
-            *reinterpret_cast<typename E::V4*>(dkp + (int64_t)row * a.k_ss + d) = kvv;
-            typename E::V2 u0 = E::cvt2(dv[gk][db][4 * r4 + 0], dv[gk][db][4 * r4 + 1]);
-            typename E::V2 u1 = E::cvt2(dv[gk][db][4 * r4 + 2], dv[gk][db][4 * r4 + 3]);
-            typename E::V4 vvv = {u0[0], u0[1], u1[0], u1[1]};
-            *reinterpret_cast<typename E::V4*>(dvp + (int64_t)row * a.v_ss + d) = vvv;
-          }
-        }
+      for (int r4 = 0; r4 < 4; r4++) {
+        typename E::V2 t0 = E::cvt2(acc[gk][db][4 * r4 + 0] * oscale, acc[gk][db][4 * r4 + 1] * oscale);
+        typename E::V2 t1 = E::cvt2(acc[gk][db][4 * r4 + 2] * oscale, acc[gk][db][4 * r4 + 3] * oscale);
+        typename E::V4 ov = {t0[0], t0[1], t1[0], t1[1]};
+        *reinterpret_cast<ACCT_LDS typename E::V4*>(obuf + l32 * OPITCH + (32 * db + 8 * r4 + 4 * g) * 2) = ov;
+      }
+    constexpr int NCH = C::CPR;
+#pragma unroll
+    for (int i = 0; i < (32 * NCH + 63) / 64; i++) {
+      const int idx = lane + 64 * i;
+      const int r = idx / NCH, ch = idx % NCH;
+      const int grow = wk0 + 32 * gk + r;
+      if (idx < 32 * NCH && grow < a.Sk) {
+        const u32x4 v = *reinterpret_cast<const ACCT_LDS u32x4*>(obuf + r * OPITCH + ch * 16);
+        *reinterpret_cast<u32x4*>(outp + (int64_t)grow * oss + ch * 8) = v;
+      }
     }
   }
 }
 
+#undef FOFF
+#undef TOFF
+#undef EDGE_PATH
+
 // ---- launchers ----------------------------------------------------------------
 template <typename T, int D, bool BIAS, bool DROP>
 static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
-  using C = TileCfg<D>;
-  const size_t smem = 4 * (size_t)C::TILEB;
   hipError_t e = hipSuccess;
   if (stages & kStageDq) {
     constexpr int QG = 1, NW = 8;
@@ -503,12 +608,15 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
     if (e != hipSuccess) return e;
   }
   if (stages & kStageDkDv) {
-    constexpr int KG = 1;
-    a.n_tiles = (a.Sk + 128 * KG - 1) / (128 * KG);
-    auto kern = fa_bwd_dkdv_kernel<T, D, KG, BIAS, DROP>;
-    e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    using CS = SwzCfg<D>;
+    constexpr size_t stageb = 2 * 64 * (size_t)CS::PITCH + 512;
+    constexpr size_t loopb = 2 * stageb + 8 * 4096 + 8 * (D >= 128 ? ACCT_PARK : 0) * 1024, epib = (size_t)8 * 32 * (CS::DB * 64 + 16);
+    const size_t smem2 = loopb > epib ? loopb : epib;
+    a.n_tiles = (a.Sk + 255) / 256;
+    auto kern = fa_bwd_dkdv_kernel<T, D, BIAS, DROP>;
+    e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem2);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((unsigned)((long long)a.n_tiles * a.B * a.N)), dim3(256), smem, st, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((long long)a.n_tiles * a.B * a.N)), dim3(512), smem2, st, a);
     e = hipGetLastError();
   }
   return e;

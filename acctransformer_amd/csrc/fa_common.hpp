@@ -98,7 +98,7 @@ struct FaArgs {
   int64_t o_sb, o_sh, o_ss;
   int64_t mask_sb;
   int64_t al_sb, al_sh, al_sq;
-  float scale, scale_log2e, inv_keep;
+  float scale, scale_log2e, inv_keep, inv_scale;
   float mask_add_raw;                  // -10000 / scale: the mask in raw q.k units
   int prev_blk, next_blk;
   int mask_kind;
@@ -194,7 +194,9 @@ ACCT_DEV void tile_dma(const T* base, int64_t row_stride, int row0, int nrows, A
   using C = SwzCfg<D>;
   constexpr int NI = ROWS / C::RPI;
   static_assert(NI % NW == 0, "tile rows must split evenly over the waves");
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));                   // addresses are re-derived per call instead of living in registers
+  const int lane = tid & 63, wave = tid >> 6;
 #pragma unroll
   for (int i = 0; i < NI / NW; i++) {
     const int inst = wave * (NI / NW) + i;
