@@ -143,7 +143,7 @@ size_t acct_fa_fwd_workspace_bytes(const acct_fa_params* p) {
 
 size_t acct_fa_bwd_workspace_bytes(const acct_fa_params* p) {
   if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0) return 0;
-  return align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + flag_bytes(p);
+  return 2 * align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + flag_bytes(p);
 }
 
 int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, size_t workspace_bytes, void* stream) {
@@ -198,9 +198,11 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
   acct::FaArgs a = make_args(p);
   a.o = const_cast<void*>(O); a.lse = const_cast<float*>(LSE);
   a.dout = dO; a.dq = dQ; a.dk = dK; a.dv = dV;
+  const size_t stat_bytes = align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256);
   a.delta = (float*)workspace;
+  a.nlse = (float*)((char*)workspace + stat_bytes);
   if (p->mask_kind == ACCT_MASK_DENSE_U8) {
-    uint8_t* flags = (uint8_t*)workspace + align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256);
+    uint8_t* flags = (uint8_t*)workspace + 2 * stat_bytes;
     a.blkflags = flags;
     if (want_dq || stages == acct::kStageDkDv) {   // the dkdv-only call re-derives the flags: the mask may have been edited since
       hipError_t e = acct::launch_mask_blocks(a, flags, p->mask_stride_b ? p->B : 1, st);

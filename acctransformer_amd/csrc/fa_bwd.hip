@@ -97,19 +97,22 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
     lq[gq] = INFINITY;                                   // rows past Sq: P = exp2(x - inf) = 0
     if (row < a.Sq) {
       lq[gq] = a.lse[(int64_t)bh * a.Sq + row] * kLog2e;
-      if (g == 0) a.delta[(int64_t)bh * a.Sq + row] = dl[gq];
+      if (g == 0) {
+        a.delta[(int64_t)bh * a.Sq + row] = dl[gq];
+        a.nlse[(int64_t)bh * a.Sq + row] = -lq[gq];        // -LSE*log2(e): the exp2 offset the dK/dV kernel adds
+      }
     }
   }
 
   // per-lane LDS offsets (tile-invariant)
   int koff[C::KS];
 #pragma unroll
-  for (int t = 0; t < C::KS; t++) koff[t] = l32 * C::PITCH + swz_off(2 * t + g, l32 & 7);
+  for (int t = 0; t < C::KS; t++) koff[t] = l32 * C::PITCH + swz_off(2 * t + g, swz3(l32));
   const int trow = 4 * g + ((lane & 15) >> 2);
   const int tchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
   int toff[C::DB];
 #pragma unroll
-  for (int db = 0; db < C::DB; db++) toff[db] = trow * C::PITCH + swz_off(4 * db + tchunk, trow) + 8 * (lane & 1);
+  for (int db = 0; db < C::DB; db++) toff[db] = trow * C::PITCH + swz_off(4 * db + tchunk, swz3(trow)) + 8 * (lane & 1);
 
   f32x16 acc[QG][C::DB];
 #pragma unroll
@@ -131,7 +134,9 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   if (j_lo <= j_hi) {
     tile_dma<T, D, 64, NW>(kp, a.k_ss, j_lo * 64, a.Sk, smem);
     tile_dma<T, D, 64, NW>(vp, a.v_ss, j_lo * 64, a.Sk, smem + TILEB);
-    dma_wait();
+    // A full wait the compiler can see: every load issued so far (Q, dO fragments included) is complete,
+    // so it places no vmcnt wait inside the loop -- such a wait would also stall on the next tile's DMA.
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
     for (int j = j_lo; j <= j_hi; j++) {
@@ -295,8 +300,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   constexpr int NW = 8;
   constexpr int BNK = 256;                          // key rows per workgroup
   constexpr int TILEB = 64 * C::PITCH;
-  constexpr int STATB = 2 * 64 * 4;                 // LSE and D of the 64 rows of a tile
-  constexpr int STAGEB = 2 * TILEB + STATB;         // one buffer: Q tile | dO tile | LSE | D
+  constexpr int STATB = 2 * 64 * 4;                 // -LSE*log2(e) and D of the 64 rows of a tile
+  constexpr int STAGEB = 2 * TILEB + STATB;         // one buffer: Q tile | dO tile | -LSE*log2(e) | D
   constexpr int PXB = 4096;                         // P of one pair and chunk: 64 lanes x 64 bytes
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 stage buffers][2 x 4 pair P buffers]
@@ -317,9 +322,6 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   const T* kp = (const T*)a.k + b * a.k_sb + h * a.k_sh;
   const T* vp = (const T*)a.v + b * a.v_sb + h * a.v_sh;
   const T* dop = (const T*)a.dout + b * a.o_sb + h * a.o_sh;
-  const float* lsep = a.lse + (int64_t)bh * a.Sq;
-  const float* delp = a.delta + (int64_t)bh * a.Sq;
-
   // visible query tiles (64 rows) of this workgroup
   const int kb_lo = k0 / 128, kb_hi = (k_end - 1) / 128;
   const int qb_lo = max(0, kb_lo - a.next_blk), qb_hi = min(a.Tr - 1, kb_hi + a.prev_blk);
@@ -376,9 +378,9 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   auto stage = [&](int i, ACCT_LDS char* sb) {
     tile_dma<T, D, 64, NW>(qp, a.q_ss, i * 64, a.Sq, sb);
     tile_dma<T, D, 64, NW>(dop, a.o_ss, i * 64, a.Sq, sb + TILEB);
-    if (wave < 2) {
+    if (wave < 2) {                                  // (pointers rebuilt from the kernel arguments: nothing to keep live)
       const int r = min(i * 64 + lane, a.Sq - 1);
-      dma4((wave == 0 ? lsep : delp) + r, sb + 2 * TILEB + wave * 256);
+      dma4((wave == 0 ? a.nlse : a.delta) + (int64_t)bh * a.Sq + r, sb + 2 * TILEB + wave * 256);
     }
   };
 
@@ -401,14 +403,22 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 
   if (i_lo <= i_hi) {
     stage(i_lo, smem);
-    dma_wait();
+    // A full wait the compiler can see: the stationary fragments loaded above are complete, so it places
+    // no vmcnt wait inside the loop -- such a wait would also stall on the next tile's DMA.
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
     // The K role runs one chunk behind the V role: in step n the V role recomputes P of chunk n,
     // publishes it and accumulates dV; the K role picks up P of chunk n-1.  One barrier per step,
     // nothing is carried across it in registers.
     const int c_lo = 2 * i_lo, c_hi = 2 * i_hi + 1;
+#ifdef ACCT_TRACE
+#define TR(k) if (blockIdx.x == ACCT_TRACE && lane == 0 && n - c_lo < 96) ((unsigned long long*)((char*)a.delta + 2 * (size_t)a.B * a.N * a.Sq * 4))[((wave * 96) + (n - c_lo)) * 8 + (k)] = __builtin_amdgcn_s_memtime()
+#else
+#define TR(k)
+#endif
     for (int n = c_lo; n <= c_hi + 1; n++) {
+      TR(0);
       if ((n & 1) && (n >> 1) < i_hi) stage((n >> 1) + 1, smem + ((((n >> 1) + 1 - i_lo) & 1) * STAGEB));
       const int cidx = krole ? n - 1 : n;             // the chunk this wave works on in this step
       if (cidx >= c_lo && cidx <= c_hi) {
@@ -424,12 +434,12 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
           asm volatile("" : "+v"(ln));
           int foff4[4];                               // row-major fragment of k-step t: row l32, chunk 2t + g
 #pragma unroll
-          for (int t = 0; t < 4; t++) foff4[t] = (ln & 31) * C::PITCH + swz_off(2 * t + (ln >> 5), ln & 7);
+          for (int t = 0; t < 4; t++) foff4[t] = (ln & 31) * C::PITCH + swz_off(2 * t + (ln >> 5), swz3(ln & 31));
           const int trow = 4 * (ln >> 5) + ((ln & 15) >> 2);
           const int tchunk = 2 * ((ln >> 4) & 1) + ((ln & 3) >> 1);
           int toff2[2];                               // transposed fragment of d block db
 #pragma unroll
-          for (int db = 0; db < 2; db++) toff2[db] = trow * C::PITCH + swz_off(4 * db + tchunk, trow) + 8 * (ln & 1);
+          for (int db = 0; db < 2; db++) toff2[db] = trow * C::PITCH + swz_off(4 * db + tchunk, swz3(trow)) + 8 * (ln & 1);
           ACCT_LDS char* qbuf = smem + (((cidx >> 1) - i_lo) & 1) * STAGEB;
           ACCT_LDS char* dobuf = qbuf + TILEB;
           const ACCT_LDS float* lbuf = (const ACCT_LDS float*)(qbuf + 2 * TILEB);
@@ -442,18 +452,26 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 #pragma unroll
             for (int r = 0; r < 16; r++) t0[gk][r] = 0.f;
           {
+            // software pipeline: the fragments of k-step t+1 are requested before the MFMAs of k-step t
             const ACCT_LDS char* abuf = (krole ? dobuf : qbuf) + c * 32 * C::PITCH;
+            V8 af = lds_read_frag<T>(abuf + FOFF(0));
+            V8 b1 = (0 >= C::KS - PARK) ? *reinterpret_cast<const ACCT_LDS V8*>(park) : bf[1][0];
 #pragma unroll
             for (int t = 0; t < C::KS; t++) {
-              const V8 af = lds_read_frag<T>(abuf + FOFF(t));
-#pragma unroll
-              for (int gk = 0; gk < 2; gk++) {                                             // S[q, key] or dP[q, key]
-                const V8 b = (gk == 1 && t >= C::KS - PARK) ? *reinterpret_cast<const ACCT_LDS V8*>(park + (t - (C::KS - PARK)) * 1024)
-                                                            : bf[gk][t];
-                t0[gk] = E::mfma(af, b, t0[gk]);
+              V8 afn = af, b1n = b1;
+              if (t + 1 < C::KS) {
+                afn = lds_read_frag<T>(abuf + FOFF(t + 1));
+                b1n = (t + 1 >= C::KS - PARK) ? *reinterpret_cast<const ACCT_LDS V8*>(park + (t + 1 - (C::KS - PARK)) * 1024) : bf[1][t + 1];
               }
+              __builtin_amdgcn_sched_barrier(0);
+              t0[0] = E::mfma(af, bf[0][t], t0[0]);                                         // S[q, key] or dP[q, key]
+              t0[1] = E::mfma(af, b1, t0[1]);
+              __builtin_amdgcn_sched_barrier(0);
+              af = afn;
+              b1 = b1n;
             }
           }
+          TR(1);
           V8 bfr[2][2];                               // B fragments of the second product: P (V role) or dS (K role)
           if (!krole) {
             if (EDGE_PATH) {
@@ -498,7 +516,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
                   const f32x4 lv = *reinterpret_cast<const ACCT_LDS f32x4*>(lbuf + 32 * c + 16 * hh + 8 * r4 + 4 * g);
 #pragma unroll
                   for (int e = 0; e < 4; e++) {
-                    p[4 * r4 + e] = fast_exp2(__builtin_fmaf(t0[gk][8 * hh + 4 * r4 + e], a.scale_log2e, lv[e] * -kLog2e));
+                    p[4 * r4 + e] = fast_exp2(__builtin_fmaf(t0[gk][8 * hh + 4 * r4 + e], a.scale_log2e, lv[e]));
                     pd[4 * r4 + e] = p[4 * r4 + e];
                     if (DROP) {
                       const int q_c = min(qc0 + 16 * hh + 8 * r4 + 4 * g + e, a.Sq - 1);
@@ -536,6 +554,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
               }
             }
           }
+          TR(2);
           // dV^T += dO^T P (V role) ; dK^T += Q^T dS (K role): contract over the 32 query rows of the chunk
           const ACCT_LDS char* tb = (krole ? qbuf : dobuf) + c * 32 * C::PITCH;
 #pragma unroll
@@ -549,9 +568,13 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
             }
         }
       }
+      TR(3);
       dma_wait();                                     // a tile requested at the top of this step has landed
+      TR(4);
       __syncthreads();
+      TR(5);
     }
+#undef TR
   }
 
   // ---- epilogue: dV (V role) / scale * dK (K role), transposed through the wave's own LDS region ----

@@ -87,7 +87,8 @@ ACCT_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 struct FaArgs {
   const void* q; const void* k; const void* v;
   void* o; float* lse;                 // fwd outputs / bwd inputs
-  const void* dout; void* dq; void* dk; void* dv; float* delta;   // bwd only
+  const void* dout; void* dq; void* dk; void* dv;                // bwd only
+  float* delta; float* nlse;           // bwd workspace: D = rowsum(dO*O) and -LSE*log2(e), [B,N,Sq] each
   const uint8_t* mask; const uint8_t* drop; const void* alibi;
   const uint8_t* blkflags;             // [MB, Tr, Tc] block classes of a dense mask
   int B, N, Sq, Sk;
@@ -170,11 +171,16 @@ ACCT_DEV void tile_store(ACCT_LDS char* buf, const u32x4 (&reg)[TileCfg<D, NT>::
 
 // ---- swizzled LDS tiles filled by direct-to-LDS loads --------------------------
 // Row pitch is a power of two (no padding, as the DMA writes 64 consecutive 16-byte
-// slots per wave instruction); the 16-byte chunk c of row r lives in slot c ^ (r & 7).
-// Eight consecutive rows then put one logical chunk into eight different 4-bank
-// groups, so both the 16-byte fragment reads (lane = row) and the transposed
-// 8-byte reads are free of bank conflicts.
+// slots per wave instruction); the 16-byte chunk c of row r lives in slot c ^ swz3(r),
+// swz3(r) = ((r & 3) << 1) | ((r >> 2) & 1).  Eight consecutive rows put one logical
+// chunk into eight different slots (16-byte fragment reads, lane = row, conflict
+// free), and four consecutive rows put one 32-byte chunk PAIR into four different
+// pairs of slots, which is what the transposed 8-byte reads (4 rows x 32 bytes per
+// 16 lanes) need.  With the plain r & 7 swizzle rows r and r^1 share a pair and every
+// transposed read takes a two-way bank conflict.
 #define ACCT_GLB __attribute__((address_space(1)))
+
+ACCT_DEV int swz3(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
 
 template <int D> struct SwzCfg {
   static constexpr int KS = D / 16;             // 16-wide k-steps across the head dim
@@ -201,7 +207,7 @@ ACCT_DEV void tile_dma(const T* base, int64_t row_stride, int row0, int nrows, A
   for (int i = 0; i < NI / NW; i++) {
     const int inst = wave * (NI / NW) + i;
     const int r = inst * C::RPI + lane / C::CH;
-    const int lc = min((lane % C::CH) ^ (r & 7), C::CPR - 1);
+    const int lc = min((lane % C::CH) ^ swz3(r), C::CPR - 1);
     const int grow = min(row0 + r, nrows - 1);
     const T* src = base + (int64_t)grow * row_stride + lc * 8;
     // Issued as inline assembly on purpose: the compiler then does not order every later LDS read
@@ -216,7 +222,7 @@ ACCT_DEV void tile_dma(const T* base, int64_t row_stride, int row0, int nrows, A
 // all of this wave's direct-to-LDS loads have landed
 ACCT_DEV void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
-// byte offset of logical chunk `lc` in a row whose (row & 7) is `swz`
+// byte offset of logical chunk `lc` in a row whose swz3(row) is `swz`
 ACCT_DEV int swz_off(int lc, int swz) { return (lc ^ swz) << 4; }
 
 }  // namespace acct

@@ -65,12 +65,12 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   // ---- per-lane LDS offsets (tile-invariant) ----
   int koff[C::KS];                                          // K fragment of k-step t: row l32, chunk 2t + g
 #pragma unroll
-  for (int t = 0; t < C::KS; t++) koff[t] = l32 * C::PITCH + swz_off(2 * t + g, l32 & 7);
+  for (int t = 0; t < C::KS; t++) koff[t] = l32 * C::PITCH + swz_off(2 * t + g, swz3(l32));
   const int trow = 4 * g + ((lane & 15) >> 2);              // transposed reads: row within an 8-row group
   const int tchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
   int voff[C::DB];                                          // V^T fragment of d block db
 #pragma unroll
-  for (int db = 0; db < C::DB; db++) voff[db] = trow * C::PITCH + swz_off(4 * db + tchunk, trow) + 8 * (lane & 1);
+  for (int db = 0; db < C::DB; db++) voff[db] = trow * C::PITCH + swz_off(4 * db + tchunk, swz3(trow)) + 8 * (lane & 1);
 
   f32x16 o[QG][C::DB];
   float m[QG], lsum[QG];
@@ -88,6 +88,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   // bias is added, in which case they are converted to log2 units first.
   const float cmul = BIAS ? 1.0f : a.scale_log2e;
   const float madd = BIAS ? kMaskFill * kLog2e : a.mask_add_raw;   // the additive -10000 in the units of s
+  const float lazy_thr = 8.0f / cmul;                              // 8 octaves, in the units of s
   const int mb = a.mask_sb ? b : 0;
   const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
   const uint8_t* dropp = DROP ? a.drop + ((int64_t)bh * a.Sq) * a.Sk : nullptr;
@@ -100,7 +101,9 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   if (j_lo <= j_hi) {
     tile_dma<T, D, 64, NW>(kp, a.k_ss, j_lo * 64, a.Sk, smem);
     tile_dma<T, D, 64, NW>(vp, a.v_ss, j_lo * 64, a.Sk, smem + TILEB);
-    dma_wait();
+    // A full wait the compiler can see: every load issued so far (Q fragments included) is complete, so
+    // it places no vmcnt wait inside the loop -- such a wait would also stall on the next tile's DMA.
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
     for (int j = j_lo; j <= j_hi; j++) {
@@ -193,8 +196,13 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
 #pragma unroll
             for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[gq][c][r]);
           mx = pair_max(mx);
-          const float m_new = fmaxf(m[gq], mx);
-          const float alpha = fast_exp2((m[gq] - m_new) * cmul);
+          // Lazy running max: it only moves when a score beats it by more than 2^8 in probability
+          // terms.  Until then P = exp2(s - m) may reach 256 instead of 1 (harmless in fp16/bf16 and in
+          // the fp32 sums; O = acc / l and LSE = m + ln l are unchanged), and the O rescale below is
+          // skipped for almost every tile after the first.
+          const bool grow = mx > m[gq] + lazy_thr;
+          const float m_new = grow ? mx : m[gq];
+          const float alpha = grow ? fast_exp2((m[gq] - m_new) * cmul) : 1.0f;
           const float mc = m_new * cmul;
           m[gq] = m_new;
           float rs = 0.f;

@@ -14,7 +14,70 @@ namespace acct {
 
 constexpr uint8_t kBlkAllMasked = 3;   // provisional: resolved to skip or apply below
 
-// one workgroup per (mask batch, q block); thread t scans 64 columns of row t/2
+// Fast path (Sk and the mask pointers 16-byte aligned, at most 64 column blocks per pass): one
+// workgroup of 1024 threads per (mask batch, q block); thread t owns the 16-byte piece t%8 of row
+// t/8 of every 128x128 block, so a block is one 16-byte load per thread and many blocks are in
+// flight at once.  Per-block "any masked" / "any unmasked" bits are gathered in two 64-bit masks
+// and reduced once at the end.
+__global__ void __launch_bounds__(1024) fa_mask_blocks_vec_kernel(const FaArgs a, uint8_t* flags) {
+  __shared__ unsigned long long s_m, s_u;
+  const int qb = blockIdx.x % a.Tr, mb = blockIdx.x / a.Tr;
+  const int tid = threadIdx.x, row = qb * 128 + (tid >> 3), c0 = (tid & 7) * 16;
+  const uint8_t* mrow = a.mask + (int64_t)mb * a.mask_sb + (int64_t)min(row, a.Sq - 1) * a.Sk;
+  uint8_t* frow = flags + ((int64_t)mb * a.Tr + qb) * a.Tc;
+  int lo = max(0, qb - a.prev_blk), hi = min(a.Tc - 1, qb + a.next_blk);
+  if (a.row_prefix) hi = min(hi, ((qb * 128 / a.row_prefix + 1) * a.row_prefix - 1) / 128);
+  for (int kvb = tid; kvb < a.Tc; kvb += 1024)
+    if (kvb < lo || kvb > hi) frow[kvb] = kBlkClean;
+  bool row_unmasked = false;
+  for (int base = lo; base <= hi; base += 64) {        // 64 column blocks per pass
+    if (tid == 0) { s_m = 0; s_u = 0; }
+    __syncthreads();
+    unsigned long long bm = 0, bu = 0;
+    const int n = min(64, hi - base + 1);
+    if (row < a.Sq) {
+#pragma unroll 8
+      for (int i = 0; i < n; i++) {
+        const int kv = (base + i) * 128 + c0;
+        if (kv < a.Sk) {                                // Sk % 16 == 0: a piece is entirely inside or outside
+          const u32x4 v = *reinterpret_cast<const u32x4*>(mrow + kv);
+          // a byte is zero iff (x - 0x01010101) & ~x & 0x80808080 has its top bit set
+          bool has_zero = false, has_nonzero = false;
+#pragma unroll
+          for (int w = 0; w < 4; w++) {
+            has_nonzero |= v[w] != 0;
+            has_zero |= ((v[w] - 0x01010101u) & ~v[w] & 0x80808080u) != 0;
+          }
+          if (has_nonzero) bm |= 1ull << i;
+          if (has_zero) bu |= 1ull << i;
+        }
+      }
+    }
+    row_unmasked |= bu != 0;
+    // wave-level OR, then one LDS atomic per wave
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      bm |= __shfl_xor(bm, off);
+      bu |= __shfl_xor(bu, off);
+    }
+    if ((tid & 63) == 0) { atomicOr(&s_m, bm); atomicOr(&s_u, bu); }
+    __syncthreads();
+    for (int i = tid; i < n; i += 1024) {
+      const bool blk_m = (s_m >> i) & 1, blk_u = (s_u >> i) & 1;
+      frow[base + i] = !blk_m ? kBlkClean : (!blk_u ? kBlkAllMasked : kBlkApply);
+    }
+    __syncthreads();
+  }
+  // a row is covered if any of its 8 threads saw an unmasked byte
+  row_unmasked |= (bool)__shfl_xor((int)row_unmasked, 1);
+  row_unmasked |= (bool)__shfl_xor((int)row_unmasked, 2);
+  row_unmasked |= (bool)__shfl_xor((int)row_unmasked, 4);
+  const int rows_ok = __syncthreads_and(row >= a.Sq || row_unmasked);
+  for (int kvb = lo + tid; kvb <= hi; kvb += 1024)
+    if (frow[kvb] == kBlkAllMasked) frow[kvb] = rows_ok ? kBlkSkip : kBlkApply;
+}
+
+// Generic path (any alignment): one workgroup per (mask batch, q block); thread t scans 64 columns of row t/2
 __global__ void __launch_bounds__(256) fa_mask_blocks_kernel(const FaArgs a, uint8_t* flags) {
   const int qb = blockIdx.x % a.Tr, mb = blockIdx.x / a.Tr;
   const int tid = threadIdx.x, row = qb * 128 + (tid >> 1), c0 = (tid & 1) * 64;
@@ -52,7 +115,9 @@ __global__ void __launch_bounds__(256) fa_mask_blocks_kernel(const FaArgs a, uin
 }
 
 hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, int MB, hipStream_t st) {
-  hipLaunchKernelGGL(fa_mask_blocks_kernel, dim3((unsigned)(MB * a.Tr)), dim3(256), 0, st, a, flags);
+  const bool vec = (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 15) == 0;
+  if (vec) hipLaunchKernelGGL(fa_mask_blocks_vec_kernel, dim3((unsigned)(MB * a.Tr)), dim3(1024), 0, st, a, flags);
+  else hipLaunchKernelGGL(fa_mask_blocks_kernel, dim3((unsigned)(MB * a.Tr)), dim3(256), 0, st, a, flags);
   return hipGetLastError();
 }
 

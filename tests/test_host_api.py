@@ -79,7 +79,7 @@ def test_null_outputs_and_workspace_sizes():
     assert lib.acct_fa_fwd(ctypes.byref(p), None, None, None, 0, None) == -1
     assert lib.acct_fa_fwd(None, None, None, None, 0, None) == -1
     assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p)) == 0
-    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p)) == 1 * 2 * 128 * 4
+    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p)) == 2 * (1 * 2 * 128 * 4)
     m = torch.zeros(1, 128, 128, dtype=torch.uint8)
     q = torch.zeros(2, 2, 128, 128, dtype=torch.float16)
     p2 = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m)
@@ -88,7 +88,7 @@ def test_null_outputs_and_workspace_sizes():
     addr = (ctypes.addressof(raw) + 63) // 64 * 64
     # backward without its workspace is refused before any launch
     assert lib.acct_fa_bwd(ctypes.byref(p2), *([addr] * 6), None, 0, None) == -7
-    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p2)) == 2 * 2 * 128 * 4 + 256
+    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p2)) == 2 * (2 * 2 * 128 * 4) + 256
 
 
 def test_no_cpu_fallback():
