@@ -131,6 +131,9 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   const bool drop_vec = DROP && (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 3) == 0;
   const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
+  TileDma<T, D, 64, NW> kdma, vdma;
+  kdma.plan(a.k_ss);
+  vdma.plan(a.v_ss);
   if (j_lo <= j_hi) {
     tile_dma<T, D, 64, NW>(kp, a.k_ss, j_lo * 64, a.Sk, smem);
     tile_dma<T, D, 64, NW>(vp, a.v_ss, j_lo * 64, a.Sk, smem + TILEB);
@@ -144,8 +147,14 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
       ACCT_LDS char* kbuf = smem + buf * 2 * TILEB;
       ACCT_LDS char* vbuf = kbuf + TILEB;
       if (j < j_hi) {
-        tile_dma<T, D, 64, NW>(kp, a.k_ss, (j + 1) * 64, a.Sk, smem + (buf ^ 1) * 2 * TILEB);
-        tile_dma<T, D, 64, NW>(vp, a.v_ss, (j + 1) * 64, a.Sk, smem + (buf ^ 1) * 2 * TILEB + TILEB);
+        ACCT_LDS char* nb = smem + (buf ^ 1) * 2 * TILEB;
+        if ((j + 2) * 64 <= a.Sk) {
+          kdma.issue(kp, a.k_ss, (j + 1) * 64, nb);
+          vdma.issue(vp, a.v_ss, (j + 1) * 64, nb + TILEB);
+        } else {                                            // ragged last tile: clamped rows
+          tile_dma<T, D, 64, NW>(kp, a.k_ss, (j + 1) * 64, a.Sk, nb);
+          tile_dma<T, D, 64, NW>(vp, a.v_ss, (j + 1) * 64, a.Sk, nb + TILEB);
+        }
       }
       const int kv0 = j * 64;
       const int kvb = j >> 1;
@@ -375,9 +384,15 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 
   // stage q tile i into buffer `sb`: Q and dO by 16-byte DMA (2 instructions per wave each),
   // LSE (wave 0) and D (wave 1) by 4-byte DMA; rows past Sq repeat the last row
+  // (addresses are re-derived per call here: this kernel has no registers to spare for a TileDma plan)
   auto stage = [&](int i, ACCT_LDS char* sb) {
-    tile_dma<T, D, 64, NW>(qp, a.q_ss, i * 64, a.Sq, sb);
-    tile_dma<T, D, 64, NW>(dop, a.o_ss, i * 64, a.Sq, sb + TILEB);
+    if ((i + 1) * 64 <= a.Sq) {
+      TileDma<T, D, 64, NW>::issue_direct(qp, a.q_ss, i * 64, sb);
+      TileDma<T, D, 64, NW>::issue_direct(dop, a.o_ss, i * 64, sb + TILEB);
+    } else {                                         // ragged last tile: clamped rows
+      tile_dma<T, D, 64, NW>(qp, a.q_ss, i * 64, a.Sq, sb);
+      tile_dma<T, D, 64, NW>(dop, a.o_ss, i * 64, a.Sq, sb + TILEB);
+    }
     if (wave < 2) {                                  // (pointers rebuilt from the kernel arguments: nothing to keep live)
       const int r = min(i * 64 + lane, a.Sq - 1);
       dma4((wave == 0 ? a.nlse : a.delta) + (int64_t)bh * a.Sq + r, sb + 2 * TILEB + wave * 256);

@@ -219,6 +219,58 @@ ACCT_DEV void tile_dma(const T* base, int64_t row_stride, int row0, int nrows, A
   }
 }
 
+// The same staging with everything tile-invariant hoisted: per-lane 32-bit byte offsets are
+// computed once (plan), a tile then costs a 64-bit scalar base, and per wave instruction one m0
+// write and one global_load_lds with scalar base + vector offset -- no vector ALU work in the loop.
+// Only tiles that lie entirely inside the matrix may use it (no row clamping).
+template <typename T, int D, int ROWS, int NW>
+struct TileDma {
+  using C = SwzCfg<D>;
+  static constexpr int NI = ROWS / C::RPI;
+  static constexpr int NIW = NI / NW;              // instructions per wave and tile
+  uint32_t voff[NIW];
+  uint32_t lds0;                                   // LDS byte offset of this wave's first 1 KB slab within a tile
+  ACCT_DEV void plan(int64_t row_stride) {
+    static_assert(NI % NW == 0, "tile rows must split evenly over the waves");
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < NIW; i++) {
+      const int inst = wave * NIW + i;
+      const int r = inst * C::RPI + lane / C::CH;
+      const int lc = min((lane % C::CH) ^ swz3(r), C::CPR - 1);
+      voff[i] = (uint32_t)((r * row_stride + lc * 8) * (int64_t)sizeof(T));
+    }
+    lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(wave * NIW * 1024));
+  }
+  // plan-free variant for kernels without registers to spare: the 32-bit offsets are re-derived
+  // (a few 32-bit vector ops per instruction); rows [row0, row0 + ROWS) must exist
+  static ACCT_DEV void issue_direct(const T* base, int64_t row_stride, int row0, ACCT_LDS char* buf) {
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & 63, wave = tid >> 6;
+    const T* tile = base + (int64_t)row0 * row_stride;
+    const uint32_t dst0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)buf + (uint32_t)(wave * NIW * 1024));
+    const uint32_t rs = (uint32_t)row_stride * (uint32_t)sizeof(T);
+#pragma unroll
+    for (int i = 0; i < NIW; i++) {
+      const int r = (wave * NIW + i) * C::RPI + lane / C::CH;
+      const int lc = min((lane % C::CH) ^ swz3(r), C::CPR - 1);
+      const uint32_t voff = (uint32_t)r * rs + (uint32_t)lc * 16u;
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(tile), "s"(dst0 + i * 1024)
+                   : "memory");
+    }
+  }
+  // rows [row0, row0 + ROWS) must exist
+  ACCT_DEV void issue(const T* base, int64_t row_stride, int row0, ACCT_LDS char* buf) const {
+    const T* tile = base + (int64_t)row0 * row_stride;            // uniform: lives in scalar registers
+    const uint32_t dst0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)buf) + lds0;
+#pragma unroll
+    for (int i = 0; i < NIW; i++)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff[i]), "s"(tile), "s"(dst0 + i * 1024)
+                   : "memory");
+  }
+};
+
 // all of this wave's direct-to-LDS loads have landed
 ACCT_DEV void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 

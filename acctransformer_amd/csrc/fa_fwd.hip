@@ -98,6 +98,9 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   const bool drop_vec = DROP && (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 3) == 0;
   const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
+  TileDma<T, D, 64, NW> kdma, vdma;
+  kdma.plan(a.k_ss);
+  vdma.plan(a.v_ss);
   if (j_lo <= j_hi) {
     tile_dma<T, D, 64, NW>(kp, a.k_ss, j_lo * 64, a.Sk, smem);
     tile_dma<T, D, 64, NW>(vp, a.v_ss, j_lo * 64, a.Sk, smem + TILEB);
@@ -106,13 +109,25 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
+#ifdef ACCT_TRACE
+#define TR(k) if (blockIdx.x == ACCT_TRACE && lane == 0 && j - j_lo < 48) ((unsigned long long*)(a.lse + (size_t)a.B * a.N * a.Sq))[((wave * 48) + (j - j_lo)) * 8 + (k)] = __builtin_amdgcn_s_memtime()
+#else
+#define TR(k)
+#endif
     for (int j = j_lo; j <= j_hi; j++) {
+      TR(0);
       const int buf = (j - j_lo) & 1;
       ACCT_LDS char* kbuf = smem + buf * 2 * TILEB;
       ACCT_LDS char* vbuf = kbuf + TILEB;
       if (j < j_hi) {                                       // next tile streams into the other buffer meanwhile
-        tile_dma<T, D, 64, NW>(kp, a.k_ss, (j + 1) * 64, a.Sk, smem + (buf ^ 1) * 2 * TILEB);
-        tile_dma<T, D, 64, NW>(vp, a.v_ss, (j + 1) * 64, a.Sk, smem + (buf ^ 1) * 2 * TILEB + TILEB);
+        ACCT_LDS char* nb = smem + (buf ^ 1) * 2 * TILEB;
+        if ((j + 2) * 64 <= a.Sk) {
+          kdma.issue(kp, a.k_ss, (j + 1) * 64, nb);
+          vdma.issue(vp, a.v_ss, (j + 1) * 64, nb + TILEB);
+        } else {                                            // ragged last tile: clamped rows
+          tile_dma<T, D, 64, NW>(kp, a.k_ss, (j + 1) * 64, a.Sk, nb);
+          tile_dma<T, D, 64, NW>(vp, a.v_ss, (j + 1) * 64, a.Sk, nb + TILEB);
+        }
       }
       const int kv0 = j * 64;
       const int kvb = j >> 1;
@@ -127,6 +142,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
       } else if (a.mask_kind == kMaskTile) {
         apply_mask = wqb == kvb;
       }
+      TR(1);
       if (act) {
         // ---- S^T = K Q^T : s[gq][c] is the 32(kv) x 32(q) tile of kv chunk c ----
         f32x16 s[QG][2];
@@ -149,6 +165,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
 #pragma unroll
               for (int gq = 0; gq < QG; gq++) s[gq][c] = E::mfma(kf[c][t], qf[gq][t], s[gq][c]);
         }
+        TR(2);
         // element (gq, c, r): q = wq0 + 32 gq + l32 ; kv = kv0 + 32 c + 8 (r/4) + 4 g + r%4
         const bool edge = apply_mask || (causal && (kv0 + 63 > wq0)) || (kv0 + 64 > a.Sk);
         typename E::V8 pf[QG][2][2];
@@ -244,6 +261,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
               for (int r = 0; r < 16; r++) o[gq][db][r] *= alpha;
           }
         }
+        TR(3);
         // ---- O^T += V^T P^T ----
 #pragma unroll
         for (int c = 0; c < 2; c++)
@@ -257,9 +275,13 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
               for (int gq = 0; gq < QG; gq++) o[gq][db] = E::mfma(vf, pf[gq][c][hh], o[gq][db]);
             }
       }
+      TR(4);
       dma_wait();
+      TR(5);
       __syncthreads();
+      TR(6);
     }
+#undef TR
   }
 
   // ---- epilogue: O = O^T / l, LSE = m + ln l.  Each wave transposes its rows through its own
