@@ -206,6 +206,17 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
                 const float p = fast_exp2(__builtin_fmaf(s[gq][r], a.scale_log2e, -lq[gq]));
                 ds[r] = p * (dp[gq][r] - dl[gq]);
               }
+            } else if (!apply_mask && !BIAS && !DROP) {
+              // causal diagonal and/or ragged key tail only: P of a hidden key is exactly 0 (with the
+              // additive mask it underflows to the same value), one compare and select per element
+              int vis = a.Sk - 1 - kv0 - 32 * c - 4 * g;         // last visible key, relative to this lane's first
+              if (causal) vis = min(vis, qrow - kv0 - 32 * c - 4 * g);
+#pragma unroll
+              for (int r = 0; r < 16; r++) {
+                float p = fast_exp2(__builtin_fmaf(s[gq][r], a.scale_log2e, -lq[gq]));
+                if (8 * (r >> 2) + (r & 3) > vis) p = 0.f;
+                ds[r] = p * (dp[gq][r] - dl[gq]);
+              }
             } else {
 #pragma unroll
               for (int r4 = 0; r4 < 4; r4++) {
@@ -489,7 +500,22 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
           TR(1);
           V8 bfr[2][2];                               // B fragments of the second product: P (V role) or dS (K role)
           if (!krole) {
-            if (EDGE_PATH) {
+            if (EDGE_PATH && !BIAS && !DROP && !apply_mask) {
+              // causal diagonal / ragged ends only: hidden entries are removed outright (their
+              // probability is exactly 0 with the additive mask too); one compare and select each
+#pragma unroll
+              for (int gk = 0; gk < 2; gk++) {
+                const int kv = wk0 + 32 * gk + l32;
+                int lo = causal ? kv - qc0 - 4 * g : -64;       // chunk rows below it come before the key
+                int hi = a.Sq - 1 - qc0 - 4 * g;                // last query row that exists
+                if (kv >= a.Sk) hi = -64;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                  const int cr = 8 * (r >> 2) + (r & 3);
+                  if (cr < lo || cr > hi) t0[gk][r] = -INFINITY;
+                }
+              }
+            } else if (EDGE_PATH) {
               // side inputs and range limits are folded into the raw scores in place: +bias/scale,
               // -10000/scale where masked, -inf where the key or the query row does not exist.
               // Uniform 64-bit row bases + 32-bit per-lane offsets keep this path light on registers.

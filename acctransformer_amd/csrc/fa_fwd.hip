@@ -187,24 +187,39 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
               }
           }
           if (edge) {
+            if (apply_mask) {
 #pragma unroll
-            for (int c = 0; c < 2; c++)
+              for (int c = 0; c < 2; c++)
 #pragma unroll
-              for (int r4 = 0; r4 < 4; r4++) {
-                const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
-                uint32_t mbits = 0;
-                if (apply_mask) {
+                for (int r4 = 0; r4 < 4; r4++) {
+                  const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
+                  uint32_t mbits;
                   if (a.mask_kind == kMaskDense) mbits = load_u8x4(maskp + (int64_t)qrow_c * a.Sk, kv, a.Sk, mask_vec);
                   else mbits = load_u8x4(maskp + (qrow_c & 127) * 128, kv & 127, 128, mask_vec);
-                }
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                  float x = s[gq][c][4 * r4 + e];
-                  if (((mbits >> (8 * e)) & 0xffu) || (causal && kv + e > qrow)) x += madd;
-                  if (kv + e >= a.Sk) x = -INFINITY;
-                  s[gq][c][4 * r4 + e] = x;
+                  for (int e = 0; e < 4; e++)
+                    if ((mbits >> (8 * e)) & 0xffu) s[gq][c][4 * r4 + e] += madd;
                 }
-              }
+            }
+            if (causal && kv0 + 63 > wq0 + 32 * gq) {
+              // Keys after the query are removed outright: with the additive mask their probability
+              // underflows to exactly 0 as well (the diagonal key is always visible), so the result
+              // is the same bit for bit at a third of the vector instructions.
+              const int dl = qrow - kv0 - 4 * g;
+#pragma unroll
+              for (int c = 0; c < 2; c++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                  if (32 * c + 8 * (r >> 2) + (r & 3) > dl) s[gq][c][r] = -INFINITY;
+            }
+            if (kv0 + 64 > a.Sk) {                             // ragged key tail
+              const int lim = a.Sk - kv0 - 4 * g;
+#pragma unroll
+              for (int c = 0; c < 2; c++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                  if (32 * c + 8 * (r >> 2) + (r & 3) >= lim) s[gq][c][r] = -INFINITY;
+            }
           }
           // ---- online softmax for query row qrow ----
           float mx = s[gq][0][0];
@@ -320,6 +335,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
     }
   }
 }
+
 
 template <typename T, int D, int QG, int NW, bool BIAS, bool DROP>
 static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
