@@ -54,8 +54,9 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, g = lane >> 5;
   const int BH = a.B * a.N;
-  const int bh = blockIdx.x % BH;
-  const int qt = a.n_tiles - 1 - (int)(blockIdx.x / BH);
+  int bh, rank;
+  wg_map(blockIdx.x, BH, a.n_tiles, bh, rank);
+  const int qt = a.n_tiles - 1 - rank;
   const int b = bh / a.N, h = bh % a.N;
   const int q0 = qt * BM;
   const int wq0 = q0 + wave * 32 * QG;
@@ -331,8 +332,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   const int pair = wave & 3;
   const bool krole = wave >= 4;                     // false: V role (S, P, dV); true: K role (dP, dS, dK)
   const int BH = a.B * a.N;
-  const int bh = blockIdx.x % BH;
-  const int kt = (int)(blockIdx.x / BH);            // causal: the first key tiles are the heaviest
+  int bh, kt;                                       // causal: the first key tiles are the heaviest
+  wg_map(blockIdx.x, BH, a.n_tiles, bh, kt);
   const int b = bh / a.N, h = bh % a.N;
   const int k0 = kt * BNK;
   const int wk0 = k0 + pair * 64;                   // first key row of this pair

@@ -110,6 +110,24 @@ struct FaArgs {
 enum : int { kMaskNone = 0, kMaskDense = 1, kMaskTile = 3, kMaskCausal = 4 };
 enum : uint8_t { kBlkClean = 0, kBlkApply = 1, kBlkSkip = 2 };
 
+// Workgroup id -> (batch*head, launch rank of the tile; rank 0 is launched first).  Workgroups are
+// handed to the 8 XCDs round robin (id % 8), each XCD with its own L2.  With many heads the plain
+// "head fastest" order gives every CU of an XCD a different head and nothing is shared; instead the
+// heads of an XCD are taken 8 at a time and all tiles of those 8 heads are launched together, so
+// that the workgroups streaming the same K/V (or Q/dO) rows run side by side on one L2.
+ACCT_DEV void wg_map(int id, int BH, int n_tiles, int& bh, int& rank) {
+  if (BH > 64 && (BH & 63) == 0) {
+    const int xcd = id & 7, slot = id >> 3;
+    const int per_group = 8 * n_tiles;
+    const int grp = slot / per_group, r = slot - grp * per_group;
+    rank = r >> 3;
+    bh = xcd + 8 * (grp * 8 + (r & 7));
+  } else {
+    bh = id % BH;
+    rank = id / BH;
+  }
+}
+
 // four consecutive mask / dropout bytes starting at column kv of a row
 ACCT_DEV uint32_t load_u8x4(const uint8_t* row, int kv, int limit, bool vec_ok) {
   if (vec_ok && kv + 4 <= limit) return *reinterpret_cast<const uint32_t*>(row + kv);

@@ -30,8 +30,9 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, g = lane >> 5;
   const int BH = a.B * a.N;
-  const int bh = blockIdx.x % BH;
-  const int qt = a.n_tiles - 1 - (int)(blockIdx.x / BH);   // heaviest (latest) causal tiles first
+  int bh, rank;
+  wg_map(blockIdx.x, BH, a.n_tiles, bh, rank);
+  const int qt = a.n_tiles - 1 - rank;                      // heaviest (latest) causal tiles first
   const int b = bh / a.N, h = bh % a.N;
   const int q0 = qt * BM;
   const int wq0 = q0 + wave * 32 * QG;                      // first query row of this wave
