@@ -124,6 +124,13 @@ size_t flag_bytes(const acct_fa_params* p) {
   return align_up(MB * (size_t)((p->Sq + 127) / 128) * (size_t)((p->Sk + 127) / 128), 256);
 }
 
+// per-key-column bitmaps of the mixed blocks of a dense mask (backward only): 16 bytes per (q block, key)
+size_t colbit_bytes(const acct_fa_params* p) {
+  if (p->mask_kind != ACCT_MASK_DENSE_U8) return 0;
+  const size_t MB = p->mask_stride_b ? p->B : 1;
+  return align_up(MB * (size_t)((p->Sq + 127) / 128) * (size_t)p->Sk * 16, 256);
+}
+
 int env_int(const char* name, int dflt) {
   const char* s = getenv(name);
   return s && *s ? atoi(s) : dflt;
@@ -143,7 +150,7 @@ size_t acct_fa_fwd_workspace_bytes(const acct_fa_params* p) {
 
 size_t acct_fa_bwd_workspace_bytes(const acct_fa_params* p) {
   if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0) return 0;
-  return 2 * align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + flag_bytes(p);
+  return 2 * align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + flag_bytes(p) + colbit_bytes(p);
 }
 
 int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, size_t workspace_bytes, void* stream) {
@@ -207,6 +214,12 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
     if (want_dq || stages == acct::kStageDkDv) {   // the dkdv-only call re-derives the flags: the mask may have been edited since
       hipError_t e = acct::launch_mask_blocks(a, flags, p->mask_stride_b ? p->B : 1, st);
       if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
+    }
+    if (want_dkdv) {
+      uint32_t* cbits = (uint32_t*)(flags + flag_bytes(p));
+      a.colbits = cbits;
+      hipError_t e = acct::launch_mask_colbits(a, flags, cbits, p->mask_stride_b ? p->B : 1, st);
+      if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask bitmap kernel: %s", hipGetErrorString(e));
     }
   }
   hipError_t e = acct::launch_bwd(a, p->dtype, p->D, stages, st);

@@ -42,7 +42,7 @@ ACCT_DEV typename Elem<T>::V8 pack8(const float* x) {
 // ============================================================================
 // dQ kernel (and delta): query-tile owner, structure of the forward kernel
 // ============================================================================
-template <typename T, int D, int QG, int NW, bool BIAS, bool DROP>
+template <typename T, int D, int QG, int NW, bool BIAS, bool DROP, bool MASKT>
 __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   using E = Elem<T>;
   using V8 = typename E::V8;
@@ -163,11 +163,11 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
       if (causal) act = act && (kv0 <= wq_end - 1);
       act = act && (kv0 < wkv_limit);
       bool apply_mask = false;
-      if (a.mask_kind == kMaskDense && act) {
+      if (MASKT && a.mask_kind == kMaskDense && act) {
         const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + wqb) * a.Tc + kvb];
         act = f != kBlkSkip;
         apply_mask = f == kBlkApply;
-      } else if (a.mask_kind == kMaskTile) {
+      } else if (MASKT && a.mask_kind == kMaskTile) {
         apply_mask = wqb == kvb;
       }
       const bool edge = apply_mask || (causal && (kv0 + 63 > wq0)) || (kv0 + 64 > a.Sk);
@@ -313,7 +313,9 @@ ACCT_DEV void dma4(const void* src, ACCT_LDS char* dst) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(d) : "memory");
 }
 
-template <typename T, int D, bool BIAS, bool DROP>
+// MASKT = false compiles the mask-tensor handling out (no mask, or the causal mask by index compare):
+// the hot variant must not carry that code's register pressure.
+template <typename T, int D, bool BIAS, bool DROP, bool MASKT>
 __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   using E = Elem<T>;
   using V8 = typename E::V8;
@@ -418,11 +420,11 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     if (causal) act = act && (qt0 + 63 >= wk0);
     if (a.row_prefix) act = act && (wk0 < (qt0 / a.row_prefix + 1) * a.row_prefix);
     apply_mask = false;
-    if (a.mask_kind == kMaskDense && act) {
+    if (MASKT && a.mask_kind == kMaskDense && act) {
       const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + qb) * a.Tc + wkb];
       act = f != kBlkSkip;
       apply_mask = f == kBlkApply;
-    } else if (a.mask_kind == kMaskTile) {
+    } else if (MASKT && a.mask_kind == kMaskTile) {
       apply_mask = wkb == qb;
     }
     edge = BIAS || DROP || apply_mask || (causal && (wk0 + 63 > qc0)) || (wk0 + 64 > a.Sk) || (qc0 + 32 > a.Sq);
@@ -533,13 +535,19 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
                 const int kv = wk0 + 32 * gk + l32;
                 const int kv_c = min(kv, a.Sk - 1);
                 const int mcol = a.mask_kind == kMaskDense ? kv_c : (kv_c & 127);
+                // dense mask: one word of the key column's bitmap covers the 32 rows of the chunk
+                const bool bitmap = apply_mask && a.mask_kind == kMaskDense;
+                uint32_t mw = 0;
+                if (bitmap) mw = a.colbits[((((int64_t)mb * a.Tr + (qc0 >> 7)) * a.Sk + kv_c) << 2) + ((qc0 >> 5) & 3)] >> (4 * g);
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                   const int qr = 8 * (r >> 2) + 4 * g + (r & 3);   // row within the chunk
                   const int qr_c = min(qr, qlast);
                   float x = t0[gk][r];
                   if (BIAS) x += (float)brow0[qr_c * (int)a.al_sq + kv_c] * a.inv_scale;
-                  if (apply_mask && mrow0[qr_c * mstride + mcol]) x += a.mask_add_raw;
+                  if (bitmap) {
+                    if (mw & (1u << (8 * (r >> 2) + (r & 3)))) x += a.mask_add_raw;
+                  } else if (apply_mask && mrow0[qr_c * mstride + mcol]) x += a.mask_add_raw;
                   if (causal && kv > qc0 + qr) x += a.mask_add_raw;
                   if (kv >= a.Sk || qr > qlast) x = -INFINITY;
                   t0[gk][r] = x;
@@ -665,7 +673,8 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
     constexpr size_t tiles = 4 * 64 * (size_t)CS::PITCH, stage = (size_t)NW * 32 * (CS::DB * 64 + 16);
     const size_t smem = tiles > stage ? tiles : stage;
     a.n_tiles = (a.Sq + BM - 1) / BM;
-    auto kern = fa_bwd_dq_kernel<T, D, QG, NW, BIAS, DROP>;
+    const bool mask_q = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;
+    auto kern = mask_q ? fa_bwd_dq_kernel<T, D, QG, NW, BIAS, DROP, true> : fa_bwd_dq_kernel<T, D, QG, NW, BIAS, DROP, BIAS || DROP>;
     e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)((long long)a.n_tiles * a.B * a.N)), dim3(64 * NW), smem, st, a);
@@ -678,7 +687,8 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
     constexpr size_t loopb = 2 * stageb + 8 * 4096 + 8 * (D >= 128 ? ACCT_PARK : 0) * 1024, epib = (size_t)8 * 32 * (CS::DB * 64 + 16);
     const size_t smem2 = loopb > epib ? loopb : epib;
     a.n_tiles = (a.Sk + 255) / 256;
-    auto kern = fa_bwd_dkdv_kernel<T, D, BIAS, DROP>;
+    const bool mask_t = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;
+    auto kern = mask_t ? fa_bwd_dkdv_kernel<T, D, BIAS, DROP, true> : fa_bwd_dkdv_kernel<T, D, BIAS, DROP, BIAS || DROP>;
     e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem2);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)((long long)a.n_tiles * a.B * a.N)), dim3(512), smem2, st, a);

@@ -91,6 +91,8 @@ struct FaArgs {
   float* delta; float* nlse;           // bwd workspace: D = rowsum(dO*O) and -LSE*log2(e), [B,N,Sq] each
   const uint8_t* mask; const uint8_t* drop; const void* alibi;
   const uint8_t* blkflags;             // [MB, Tr, Tc] block classes of a dense mask
+  const uint32_t* colbits;             // [MB, Tr, Sk, 4] dense mask of the 'apply' blocks packed by key column: bit r of the
+                                       // 128-bit entry = mask[128*qb + r][key] (dK/dV kernel); may be null
   int B, N, Sq, Sk;
   int Tr, Tc;                          // number of 128-row / 128-column blocks
   int64_t q_sb, q_sh, q_ss;

@@ -18,7 +18,7 @@
 
 namespace acct {
 
-template <typename T, int D, int QG, int NW, bool BIAS, bool DROP>
+template <typename T, int D, int QG, int NW, bool BIAS, bool DROP, bool MASKT>
 __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   using E = Elem<T>;
   using V8 = typename E::V8;
@@ -136,11 +136,11 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
       if (causal) act = act && (kv0 <= wq_end - 1);
       act = act && (kv0 < wkv_limit);
       bool apply_mask = false;
-      if (a.mask_kind == kMaskDense && act) {
+      if (MASKT && a.mask_kind == kMaskDense && act) {
         const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + wqb) * a.Tc + kvb];
         act = f != kBlkSkip;
         apply_mask = f == kBlkApply;
-      } else if (a.mask_kind == kMaskTile) {
+      } else if (MASKT && a.mask_kind == kMaskTile) {
         apply_mask = wqb == kvb;
       }
       TR(1);
@@ -345,7 +345,8 @@ static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
   a.n_tiles = (a.Sq + BM - 1) / BM;
   constexpr size_t tiles = 4 * 64 * (size_t)C::PITCH, stage = (size_t)NW * 32 * (C::DB * 64 + 16);
   const size_t smem = tiles > stage ? tiles : stage;
-  auto kern = fa_fwd_kernel<T, D, QG, NW, BIAS, DROP>;
+  const bool mask_t = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;
+  auto kern = mask_t ? fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, true> : fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, BIAS || DROP>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (e != hipSuccess) return e;
   const long long nblk = (long long)a.n_tiles * a.B * a.N;

@@ -114,6 +114,32 @@ __global__ void __launch_bounds__(256) fa_mask_blocks_kernel(const FaArgs a, uin
     if (frow[kvb] == kBlkAllMasked) frow[kvb] = rows_ok ? kBlkSkip : kBlkApply;
 }
 
+// Column bitmaps of the mixed ('apply') blocks for the dK/dV kernel, whose lanes own key columns: one
+// thread per key column packs the 128 rows of a block into 128 bits, so that the kernel reads one
+// 32-bit word per lane and 32-row chunk instead of 16 single bytes.
+__global__ void __launch_bounds__(128) fa_mask_colbits_kernel(const FaArgs a, const uint8_t* flags, uint32_t* out) {
+  const int kvb = blockIdx.x % a.Tc, qb = (blockIdx.x / a.Tc) % a.Tr, mb = blockIdx.x / (a.Tc * a.Tr);
+  if (flags[((int64_t)mb * a.Tr + qb) * a.Tc + kvb] != kBlkApply) return;
+  const int kv = kvb * 128 + threadIdx.x;
+  if (kv >= a.Sk) return;
+  const uint8_t* col = a.mask + (int64_t)mb * a.mask_sb + kv;
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll 8
+    for (int r = 0; r < 32; r++) {
+      const int row = qb * 128 + 32 * i + r;
+      if (row < a.Sq && col[(int64_t)row * a.Sk]) w[i] |= 1u << r;
+    }
+  u32x4 v = {w[0], w[1], w[2], w[3]};
+  *reinterpret_cast<u32x4*>(out + (((int64_t)mb * a.Tr + qb) * a.Sk + kv) * 4) = v;
+}
+
+hipError_t launch_mask_colbits(const FaArgs& a, const uint8_t* flags, uint32_t* out, int MB, hipStream_t st) {
+  hipLaunchKernelGGL(fa_mask_colbits_kernel, dim3((unsigned)(MB * a.Tr * a.Tc)), dim3(128), 0, st, a, flags, out);
+  return hipGetLastError();
+}
+
 hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, int MB, hipStream_t st) {
   const bool vec = (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 15) == 0;
   if (vec) hipLaunchKernelGGL(fa_mask_blocks_vec_kernel, dim3((unsigned)(MB * a.Tr)), dim3(1024), 0, st, a, flags);

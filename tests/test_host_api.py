@@ -88,7 +88,8 @@ def test_null_outputs_and_workspace_sizes():
     addr = (ctypes.addressof(raw) + 63) // 64 * 64
     # backward without its workspace is refused before any launch
     assert lib.acct_fa_bwd(ctypes.byref(p2), *([addr] * 6), None, 0, None) == -7
-    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p2)) == 2 * (2 * 2 * 128 * 4) + 256
+    # D and -LSE*log2e rows, block classes (padded to 256), key-column bitmaps: 16 bytes per (q block, key)
+    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p2)) == 2 * (2 * 2 * 128 * 4) + 256 + 1 * 1 * 128 * 16
 
 
 def test_no_cpu_fallback():
