@@ -126,6 +126,7 @@ size_t flag_bytes(const acct_fa_params* p) {
 
 // per-key-column bitmaps of the mixed blocks of a dense mask (backward only): 16 bytes per (q block, key)
 size_t colbit_bytes(const acct_fa_params* p) {
+  if (p->mask_kind == ACCT_MASK_TILE_U8) return 128 * 16;
   if (p->mask_kind != ACCT_MASK_DENSE_U8) return 0;
   const size_t MB = p->mask_stride_b ? p->B : 1;
   return align_up(MB * (size_t)((p->Sq + 127) / 128) * (size_t)p->Sk * 16, 256);
@@ -215,12 +216,13 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
       hipError_t e = acct::launch_mask_blocks(a, flags, p->mask_stride_b ? p->B : 1, st);
       if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
     }
-    if (want_dkdv) {
-      uint32_t* cbits = (uint32_t*)(flags + flag_bytes(p));
-      a.colbits = cbits;
-      hipError_t e = acct::launch_mask_colbits(a, flags, cbits, p->mask_stride_b ? p->B : 1, st);
-      if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask bitmap kernel: %s", hipGetErrorString(e));
-    }
+  }
+  if (want_dkdv && (p->mask_kind == ACCT_MASK_DENSE_U8 || p->mask_kind == ACCT_MASK_TILE_U8)) {
+    uint8_t* flags = (uint8_t*)workspace + 2 * stat_bytes;          // (no flags for the tile kind: flag_bytes = 0)
+    uint32_t* cbits = (uint32_t*)(flags + flag_bytes(p));
+    a.colbits = cbits;
+    hipError_t e = acct::launch_mask_colbits(a, flags, cbits, p->mask_stride_b ? p->B : 1, st);
+    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask bitmap kernel: %s", hipGetErrorString(e));
   }
   hipError_t e = acct::launch_bwd(a, p->dtype, p->D, stages, st);
   if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "backward kernels: %s", hipGetErrorString(e));

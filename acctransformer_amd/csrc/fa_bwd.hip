@@ -308,6 +308,9 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 #ifndef ACCT_PARK
 #define ACCT_PARK 6
 #endif
+#ifndef ACCT_PARK_HOT
+#define ACCT_PARK_HOT 4      // the variant without side inputs has registers for two more fragments
+#endif
 ACCT_DEV void dma4(const void* src, ACCT_LDS char* dst) {
   const uint32_t d = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst);
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(d) : "memory");
@@ -357,7 +360,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   // lane holds key row 32 gk + l32, d = 16t + 8g ..
   // The last PARK k-steps of the second key group live in a wave-private LDS slab instead of
   // registers (16 VGPRs at D = 128): that is what lets two waves share a SIMD without spilling.
-  constexpr int PARK = D >= 128 ? ACCT_PARK : 0;
+  constexpr int PARK = D >= 128 ? (MASKT ? ACCT_PARK : ACCT_PARK_HOT) : 0;
   V8 bf[2][C::KS];
   ACCT_LDS char* park = pexch + 8 * PXB + wave * (PARK * 1024) + lane * 16;
   {
@@ -503,9 +506,43 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
           TR(1);
           V8 bfr[2][2];                               // B fragments of the second product: P (V role) or dS (K role)
           if (!krole) {
-            if (EDGE_PATH && !BIAS && !DROP && !apply_mask) {
-              // causal diagonal / ragged ends only: hidden entries are removed outright (their
-              // probability is exactly 0 with the additive mask too); one compare and select each
+            if (EDGE_PATH) {
+              // Side inputs and range limits are folded into the raw scores in place, in three short
+              // passes that each keep few values live: + bias/scale; - 10000/scale where the mask bit of
+              // (row, key) is set; -inf where the key comes after the query (causal) or where the key
+              // or the query row does not exist (the probability is exactly 0 either way).
+              if (BIAS) {
+                const int qlast = a.Sq - 1 - qc0;               // last valid row, relative to the chunk
+                const T* brow0 = alibip + (int64_t)qc0 * a.al_sq;
+#pragma unroll
+                for (int gk = 0; gk < 2; gk++) {
+                  const int kv_c = min(wk0 + 32 * gk + l32, a.Sk - 1);
+#pragma unroll
+                  for (int r = 0; r < 16; r++) {
+                    const int qr_c = min(8 * (r >> 2) + 4 * g + (r & 3), qlast);
+                    t0[gk][r] += (float)brow0[qr_c * (int)a.al_sq + kv_c] * a.inv_scale;
+                    if ((r & 3) == 3) asm volatile("" ::: "memory");   // keep the loads in small batches
+                  }
+                }
+              }
+              if (MASKT && apply_mask) {
+                // one 32-bit word of the key column's bitmap covers the 32 rows of the chunk
+                const uint32_t* cb = a.mask_kind == kMaskDense
+                                         ? a.colbits + ((((int64_t)mb * a.Tr + (qc0 >> 7)) * a.Sk) << 2) + ((qc0 >> 5) & 3)
+                                         : a.colbits + ((qc0 >> 5) & 3);
+                const uint32_t addbits = __float_as_uint(a.mask_add_raw);
+#pragma unroll
+                for (int gk = 0; gk < 2; gk++) {
+                  const int kv_c = min(wk0 + 32 * gk + l32, a.Sk - 1);
+                  const uint32_t w = cb[(a.mask_kind == kMaskDense ? kv_c : (kv_c & 127)) * 4] >> (4 * g);
+#pragma unroll
+                  for (int r = 0; r < 16; r++) {
+                    // (bit ? -1 : 0) & bits(-10000/scale), added
+                    const int32_t sel = (int32_t)(w << (31 - (8 * (r >> 2) + (r & 3)))) >> 31;
+                    t0[gk][r] += __uint_as_float((uint32_t)sel & addbits);
+                  }
+                }
+              }
 #pragma unroll
               for (int gk = 0; gk < 2; gk++) {
                 const int kv = wk0 + 32 * gk + l32;
@@ -516,42 +553,6 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
                 for (int r = 0; r < 16; r++) {
                   const int cr = 8 * (r >> 2) + (r & 3);
                   if (cr < lo || cr > hi) t0[gk][r] = -INFINITY;
-                }
-              }
-            } else if (EDGE_PATH) {
-              // side inputs and range limits are folded into the raw scores in place: +bias/scale,
-              // -10000/scale where masked, -inf where the key or the query row does not exist.
-              // Uniform 64-bit row bases + 32-bit per-lane offsets keep this path light on registers.
-              const int qlast = a.Sq - 1 - qc0;                 // last valid row, relative to the chunk
-              const uint8_t* mrow0 = nullptr;
-              int mstride = 0;
-              if (apply_mask) {
-                if (a.mask_kind == kMaskDense) { mrow0 = maskp + (int64_t)qc0 * a.Sk; mstride = a.Sk; }
-                else { mrow0 = maskp + (qc0 & 127) * 128; mstride = 128; }
-              }
-              const T* brow0 = BIAS ? alibip + (int64_t)qc0 * a.al_sq : nullptr;
-#pragma unroll
-              for (int gk = 0; gk < 2; gk++) {
-                const int kv = wk0 + 32 * gk + l32;
-                const int kv_c = min(kv, a.Sk - 1);
-                const int mcol = a.mask_kind == kMaskDense ? kv_c : (kv_c & 127);
-                // dense mask: one word of the key column's bitmap covers the 32 rows of the chunk
-                const bool bitmap = apply_mask && a.mask_kind == kMaskDense;
-                uint32_t mw = 0;
-                if (bitmap) mw = a.colbits[((((int64_t)mb * a.Tr + (qc0 >> 7)) * a.Sk + kv_c) << 2) + ((qc0 >> 5) & 3)] >> (4 * g);
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                  const int qr = 8 * (r >> 2) + 4 * g + (r & 3);   // row within the chunk
-                  const int qr_c = min(qr, qlast);
-                  float x = t0[gk][r];
-                  if (BIAS) x += (float)brow0[qr_c * (int)a.al_sq + kv_c] * a.inv_scale;
-                  if (bitmap) {
-                    if (mw & (1u << (8 * (r >> 2) + (r & 3)))) x += a.mask_add_raw;
-                  } else if (apply_mask && mrow0[qr_c * mstride + mcol]) x += a.mask_add_raw;
-                  if (causal && kv > qc0 + qr) x += a.mask_add_raw;
-                  if (kv >= a.Sk || qr > qlast) x = -INFINITY;
-                  t0[gk][r] = x;
-                  if ((r & 3) == 3) asm volatile("" ::: "memory");   // keep the side-input loads in small batches
                 }
               }
             }

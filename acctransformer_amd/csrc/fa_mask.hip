@@ -135,7 +135,23 @@ __global__ void __launch_bounds__(128) fa_mask_colbits_kernel(const FaArgs a, co
   *reinterpret_cast<u32x4*>(out + (((int64_t)mb * a.Tr + qb) * a.Sk + kv) * 4) = v;
 }
 
+// the same for the compact 128x128 tile that is applied on diagonal blocks: out[key][4]
+__global__ void __launch_bounds__(128) fa_mask_tilebits_kernel(const uint8_t* tile, uint32_t* out) {
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll 8
+    for (int r = 0; r < 32; r++)
+      if (tile[(32 * i + r) * 128 + threadIdx.x]) w[i] |= 1u << r;
+  u32x4 v = {w[0], w[1], w[2], w[3]};
+  *reinterpret_cast<u32x4*>(out + threadIdx.x * 4) = v;
+}
+
 hipError_t launch_mask_colbits(const FaArgs& a, const uint8_t* flags, uint32_t* out, int MB, hipStream_t st) {
+  if (a.mask_kind == kMaskTile) {
+    hipLaunchKernelGGL(fa_mask_tilebits_kernel, dim3(1), dim3(128), 0, st, a.mask, out);
+    return hipGetLastError();
+  }
   hipLaunchKernelGGL(fa_mask_colbits_kernel, dim3((unsigned)(MB * a.Tr * a.Tc)), dim3(128), 0, st, a, flags, out);
   return hipGetLastError();
 }
