@@ -132,6 +132,17 @@ size_t colbit_bytes(const acct_fa_params* p) {
   return align_up(MB * (size_t)((p->Sq + 127) / 128) * (size_t)p->Sk * 16, 256);
 }
 
+// keep bits of the dropout mask: by query row (forward, dQ) and by key column (dK/dV)
+size_t droprow_words(const acct_fa_params* p) { return 2 * (size_t)((p->Sk + 63) / 64); }   // 32-bit words per row
+size_t droprow_bytes(const acct_fa_params* p) {
+  if (!p->drop_mask) return 0;
+  return align_up((size_t)p->B * p->N * p->Sq * droprow_words(p) * 4, 256);
+}
+size_t dropcol_bytes(const acct_fa_params* p) {
+  if (!p->drop_mask) return 0;
+  return align_up((size_t)p->B * p->N * (size_t)((p->Sq + 127) / 128) * (size_t)p->Sk * 16, 256);
+}
+
 int env_int(const char* name, int dflt) {
   const char* s = getenv(name);
   return s && *s ? atoi(s) : dflt;
@@ -145,13 +156,14 @@ const char* acct_last_error(void) { return g_err; }
 int acct_version(void) { return ACCT_FA_VERSION; }
 
 size_t acct_fa_fwd_workspace_bytes(const acct_fa_params* p) {
-  if (!p) return 0;
-  return flag_bytes(p);
+  if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0 || p->Sk <= 0) return 0;
+  return flag_bytes(p) + droprow_bytes(p);
 }
 
 size_t acct_fa_bwd_workspace_bytes(const acct_fa_params* p) {
   if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0) return 0;
-  return 2 * align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + flag_bytes(p) + colbit_bytes(p);
+  if (p->Sk <= 0) return 0;
+  return 2 * align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + flag_bytes(p) + colbit_bytes(p) + droprow_bytes(p) + dropcol_bytes(p);
 }
 
 int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, size_t workspace_bytes, void* stream) {
@@ -174,6 +186,13 @@ int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, s
     a.blkflags = (const uint8_t*)workspace;
     hipError_t e = acct::launch_mask_blocks(a, (uint8_t*)workspace, p->mask_stride_b ? p->B : 1, st);
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
+  }
+  if (p->drop_mask) {
+    uint32_t* rows = (uint32_t*)((char*)workspace + flag_bytes(p));
+    a.droprow = rows;
+    a.droprow_w = (int)droprow_words(p);
+    hipError_t e = acct::launch_drop_bits(a, rows, nullptr, st);
+    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "dropout bitmap kernel: %s", hipGetErrorString(e));
   }
   // 8 waves x 32 query rows (two waves per SIMD overlap MFMA and softmax work) once that still
   // fills the chip, else 4 waves x 32 rows for more workgroups
@@ -223,6 +242,16 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
     a.colbits = cbits;
     hipError_t e = acct::launch_mask_colbits(a, flags, cbits, p->mask_stride_b ? p->B : 1, st);
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask bitmap kernel: %s", hipGetErrorString(e));
+  }
+  if (p->drop_mask) {
+    char* base = (char*)workspace + 2 * stat_bytes + flag_bytes(p) + colbit_bytes(p);
+    uint32_t* rows = (uint32_t*)base;
+    uint32_t* cols = (uint32_t*)(base + droprow_bytes(p));
+    a.droprow = rows;
+    a.dropcol = cols;
+    a.droprow_w = (int)droprow_words(p);
+    hipError_t e = acct::launch_drop_bits(a, want_dq ? rows : nullptr, want_dkdv ? cols : nullptr, st);
+    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "dropout bitmap kernel: %s", hipGetErrorString(e));
   }
   hipError_t e = acct::launch_bwd(a, p->dtype, p->D, stages, st);
   if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "backward kernels: %s", hipGetErrorString(e));

@@ -125,11 +125,9 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 
   const int mb = a.mask_sb ? b : 0;
   const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
-  const uint8_t* dropp = DROP ? a.drop + ((int64_t)bh * a.Sq) * a.Sk : nullptr;
   const T* alibip = BIAS ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
   const bool mask_vec = a.mask_kind == kMaskDense ? (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0
                                                   : ((uintptr_t)a.mask & 3) == 0;
-  const bool drop_vec = DROP && (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 3) == 0;
   const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
   TileDma<T, D, 64, NW> kdma, vdma;
@@ -219,17 +217,18 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
                 ds[r] = p * (dp[gq][r] - dl[gq]);
               }
             } else {
+              uint32_t dw = 0xffffffffu;                        // keep bits of this row: keys kv0 + 32c .. +31
+              if (DROP) dw = a.droprow[((int64_t)bh * a.Sq + qrow_c) * a.droprow_w + 2 * j + c] >> (4 * g);
 #pragma unroll
               for (int r4 = 0; r4 < 4; r4++) {
                 const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
                 float bias[4] = {0.f, 0.f, 0.f, 0.f};
-                uint32_t mbits = 0, dbits = 0x01010101u;
+                uint32_t mbits = 0;
                 if (BIAS) load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
                 if (apply_mask) {
                   if (a.mask_kind == kMaskDense) mbits = load_u8x4(maskp + (int64_t)qrow_c * a.Sk, kv, a.Sk, mask_vec);
                   else mbits = load_u8x4(maskp + (qrow_c & 127) * 128, kv & 127, 128, mask_vec);
                 }
-                if (DROP) dbits = load_u8x4(dropp + (int64_t)qrow_c * a.Sk, kv, a.Sk, drop_vec);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                   const int r = 4 * r4 + e;
@@ -239,7 +238,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
                   float p = fast_exp2(x);
                   if (kv + e >= a.Sk) p = 0.f;
                   float dpv = dp[gq][r];
-                  if (DROP) dpv = ((dbits >> (8 * e)) & 0xffu) ? dpv * a.inv_keep : 0.f;
+                  if (DROP) dpv = ((dw >> (8 * r4 + e)) & 1u) ? dpv * a.inv_keep : 0.f;
                   ds[r] = p * (dpv - dl[gq]);
                 }
               }
@@ -396,7 +395,6 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 
   const int mb = a.mask_sb ? b : 0;
   const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
-  const uint8_t* dropp = DROP ? a.drop + ((int64_t)bh * a.Sq) * a.Sk : nullptr;
   const T* alibip = BIAS ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
 
   // stage q tile i into buffer `sb`: Q and dO by 16-byte DMA (2 instructions per wave each),
@@ -504,6 +502,12 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
             }
           }
           TR(1);
+          uint32_t dcw[2] = {0u, 0u};                 // keep bits of the chunk's 32 rows for this lane's two key columns
+          if (DROP) {
+            const uint32_t* dc = a.dropcol + ((((int64_t)bh * a.Tr + (qc0 >> 7)) * a.Sk) << 2) + ((qc0 >> 5) & 3);
+#pragma unroll
+            for (int gk = 0; gk < 2; gk++) dcw[gk] = dc[min(wk0 + 32 * gk + l32, a.Sk - 1) * 4] >> (4 * g);
+          }
           V8 bfr[2][2];                               // B fragments of the second product: P (V role) or dS (K role)
           if (!krole) {
             if (EDGE_PATH) {
@@ -569,10 +573,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
                   for (int e = 0; e < 4; e++) {
                     p[4 * r4 + e] = fast_exp2(__builtin_fmaf(t0[gk][8 * hh + 4 * r4 + e], a.scale_log2e, lv[e]));
                     pd[4 * r4 + e] = p[4 * r4 + e];
-                    if (DROP) {
-                      const int q_c = min(qc0 + 16 * hh + 8 * r4 + 4 * g + e, a.Sq - 1);
-                      pd[4 * r4 + e] = dropp[(int64_t)q_c * a.Sk + kv_c] ? p[4 * r4 + e] * a.inv_keep : 0.f;
-                    }
+                    if (DROP) pd[4 * r4 + e] = ((dcw[gk] >> (16 * hh + 8 * r4 + e)) & 1u) ? p[4 * r4 + e] * a.inv_keep : 0.f;
                   }
                 }
                 bfr[gk][hh] = pack8<T>(pd);
@@ -594,10 +595,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 #pragma unroll
                   for (int e = 0; e < 4; e++) {
                     float dpv = t0[gk][8 * hh + 4 * r4 + e];
-                    if (DROP) {
-                      const int q_c = min(qc0 + 16 * hh + 8 * r4 + 4 * g + e, a.Sq - 1);
-                      dpv = dropp[(int64_t)q_c * a.Sk + kv_c] ? dpv * a.inv_keep : 0.f;
-                    }
+                    if (DROP) dpv = ((dcw[gk] >> (16 * hh + 8 * r4 + e)) & 1u) ? dpv * a.inv_keep : 0.f;
                     ds[4 * r4 + e] = (float)ph[4 * r4 + e] * (dpv - dv4[e]);
                   }
                 }

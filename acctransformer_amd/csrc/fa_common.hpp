@@ -91,6 +91,8 @@ struct FaArgs {
   float* delta; float* nlse;           // bwd workspace: D = rowsum(dO*O) and -LSE*log2(e), [B,N,Sq] each
   const uint8_t* mask; const uint8_t* drop; const void* alibi;
   const uint8_t* blkflags;             // [MB, Tr, Tc] block classes of a dense mask
+  const uint32_t* droprow;             // [B*N*Sq, droprow_w] keep bits of the dropout mask by query row: bit k of word w = drop[row][32w+k] != 0
+  const uint32_t* dropcol;             // [B*N, Tr, Sk, 4] the same by key column: bit r of the 128-bit entry = drop[128*qb + r][key] != 0
   const uint32_t* colbits;             // [MB, Tr, Sk, 4] dense mask of the 'apply' blocks packed by key column: bit r of the
                                        // 128-bit entry = mask[128*qb + r][key] (dK/dV kernel); may be null
   int B, N, Sq, Sk;
@@ -107,6 +109,7 @@ struct FaArgs {
   int mask_kind;
   int row_prefix;                      // >0: row i sees keys j < (i/row_prefix + 1)*row_prefix only (multiple of 128)
   int n_tiles;                         // tiles along the owner dimension
+  int droprow_w;                       // 32-bit words per row of droprow: 2 * ceil(Sk / 64)
 };
 
 enum : int { kMaskNone = 0, kMaskDense = 1, kMaskTile = 3, kMaskCausal = 4 };

@@ -92,11 +92,9 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   const float lazy_thr = 8.0f / cmul;                              // 8 octaves, in the units of s
   const int mb = a.mask_sb ? b : 0;
   const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
-  const uint8_t* dropp = DROP ? a.drop + ((int64_t)bh * a.Sq) * a.Sk : nullptr;
   const T* alibip = BIAS ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
   const bool mask_vec = a.mask_kind == kMaskDense ? (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0
                                                   : ((uintptr_t)a.mask & 3) == 0;
-  const bool drop_vec = DROP && (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 3) == 0;
   const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
   TileDma<T, D, 64, NW> kdma, vdma;
@@ -249,15 +247,17 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
             }
           lsum[gq] = lsum[gq] * alpha + rs;                  // row sum BEFORE dropout
           if (DROP) {
+            // keep bits of this row and tile: word 2j + c covers keys 64j + 32c .. +31
+            const uint32_t* dr = a.droprow + ((int64_t)bh * a.Sq + qrow_c) * a.droprow_w + 2 * j;
 #pragma unroll
-            for (int c = 0; c < 2; c++)
+            for (int c = 0; c < 2; c++) {
+              const uint32_t w = dr[c] >> (4 * g);
 #pragma unroll
-              for (int r4 = 0; r4 < 4; r4++) {
-                const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
-                const uint32_t dbits = load_u8x4(dropp + (int64_t)qrow_c * a.Sk, kv, a.Sk, drop_vec);
-#pragma unroll
-                for (int e = 0; e < 4; e++) p[c][4 * r4 + e] *= ((dbits >> (8 * e)) & 0xffu) ? a.inv_keep : 0.f;
+              for (int r = 0; r < 16; r++) {
+                const int32_t sel = (int32_t)(w << (31 - (8 * (r >> 2) + (r & 3)))) >> 31;   // keep ? ~0 : 0
+                p[c][r] = __uint_as_float(__float_as_uint(p[c][r] * a.inv_keep) & (uint32_t)sel);
               }
+            }
           }
 #pragma unroll
           for (int c = 0; c < 2; c++)

@@ -14,6 +14,8 @@ hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t
 
 // classify the 128x128 blocks of a dense uint8 mask into clean / apply / skip
 hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, int MB, hipStream_t st);
+// pack the dropout mask into keep bits by query row [B*N, Sq, droprow_w] and / or by key column [B*N, Tr, Sk, 4]
+hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st);
 // pack the 'apply' blocks of a dense mask into per-key-column bitmaps [MB, Tr, Sk, 4 x u32]
 hipError_t launch_mask_colbits(const FaArgs& a, const uint8_t* flags, uint32_t* out, int MB, hipStream_t st);
 

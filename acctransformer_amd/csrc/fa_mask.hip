@@ -156,6 +156,72 @@ hipError_t launch_mask_colbits(const FaArgs& a, const uint8_t* flags, uint32_t* 
   return hipGetLastError();
 }
 
+// Dropout mask (uint8, nonzero = keep) packed into keep bits, by query row for the kernels whose lanes own
+// query rows (forward, dQ) and by key column for the dK/dV kernel.  One wave per (batch*head, 128 query
+// rows, 1024 keys): per row every lane loads the 16 bytes of keys 16*lane .. +15 (a kilobyte per wave
+// instruction keeps enough bytes in flight) and turns them into 16 bits; lane pairs form the 32-bit row words.
+//   rowbits [B*N*Sq, 2*ceil(Sk/64)] 32-bit: bit k of word w = keep[row][32w + k];
+//   colbits [B*N, Tr, Sk, 4] 32-bit: bit r of the 128-bit entry = keep[128*qb + r][key].
+__global__ void __launch_bounds__(64) fa_drop_bits_kernel(const FaArgs a, uint32_t* rowbits, uint32_t* colbits) {
+  const int nspan = (a.Sk + 1023) / 1024;
+  const int span = blockIdx.x % nspan, qb = (blockIdx.x / nspan) % a.Tr, bh = blockIdx.x / (nspan * a.Tr);
+  const int lane = threadIdx.x;
+  const int kv = span * 1024 + 16 * lane;               // first of this lane's sixteen keys
+  const bool vec = (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 15) == 0 && kv + 16 <= a.Sk;
+  const int widx = 32 * span + (lane >> 1);             // this lane pair's word within the row
+  const bool writer = rowbits && (lane & 1) == 0 && widx < a.droprow_w;
+  uint32_t* rowout = rowbits + ((int64_t)bh * a.Sq + qb * 128) * a.droprow_w + widx;
+  const uint8_t* p = a.drop + ((int64_t)bh * a.Sq + qb * 128) * a.Sk + min(kv, max(a.Sk - 16, 0));
+  const int nrow = min(128, a.Sq - qb * 128);
+  uint32_t cw[16][4];                                   // per key: four words of 32 rows, most significant bit first
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+#pragma unroll
+    for (int e = 0; e < 16; e++) cw[e][i] = 0u;
+#pragma unroll 4
+    for (int r = 0; r < 32; r++) {
+      const int rr = 32 * i + r;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (rr < nrow) {
+        if (vec) v = *reinterpret_cast<const u32x4*>(p);
+        else {
+          const uint8_t* q = a.drop + ((int64_t)bh * a.Sq + qb * 128 + rr) * a.Sk;
+#pragma unroll
+          for (int e = 0; e < 16; e++)
+            if (kv + e < a.Sk) v[e >> 2] |= (uint32_t)q[kv + e] << (8 * (e & 3));
+        }
+      }
+      p += a.Sk;                                        // per-lane pointer walks down the rows
+      uint32_t bits = 0;
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+        const uint32_t keep = ((v[e >> 2] >> (8 * (e & 3))) & 0xffu) != 0 ? 1u : 0u;
+        bits |= keep << e;
+        cw[e][i] = (cw[e][i] << 1) | keep;
+      }
+      uint32_t x = bits << (16 * (lane & 1));
+      x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xf, 0xf, true);    // lane ^ 1
+      if (writer && rr < nrow) *rowout = x;
+      rowout += a.droprow_w;
+    }
+  }
+  if (colbits) {
+#pragma unroll
+    for (int e = 0; e < 16; e++)
+      if (kv + e < a.Sk) {
+        u32x4 v = {__builtin_bitreverse32(cw[e][0]), __builtin_bitreverse32(cw[e][1]), __builtin_bitreverse32(cw[e][2]),
+                   __builtin_bitreverse32(cw[e][3])};
+        *reinterpret_cast<u32x4*>(colbits + (((int64_t)bh * a.Tr + qb) * a.Sk + kv + e) * 4) = v;
+      }
+  }
+}
+
+hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st) {
+  const long long nblk = (long long)a.B * a.N * a.Tr * ((a.Sk + 1023) / 1024);
+  hipLaunchKernelGGL(fa_drop_bits_kernel, dim3((unsigned)nblk), dim3(64), 0, st, a, rowbits, colbits);
+  return hipGetLastError();
+}
+
 hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, int MB, hipStream_t st) {
   const bool vec = (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 15) == 0;
   if (vec) hipLaunchKernelGGL(fa_mask_blocks_vec_kernel, dim3((unsigned)(MB * a.Tr)), dim3(1024), 0, st, a, flags);
