@@ -205,6 +205,22 @@ def test_padding_mask_with_dropout():
                                       drop_mask=drop, keep_prob=0.9))
 
 
+@pytest.mark.parametrize("Sq, Sk", [(300, 333), (1100, 1100), (130, 2050)])
+def test_ragged_dropout_with_random_mask(Sq, Sk):
+    # lengths off every vector width and tile edge: the keep-bit packing (16-byte loads, 1024-key spans,
+    # 32-bit row words, 128-row column entries) has a partial piece at each level
+    B, N, D = 2, 2, 128
+    q, dO = (_gen((B, N, Sq, D), s) for s in (61, 64))
+    k, v = (_gen((B, N, Sk, D), s) for s in (62, 63))
+    rng = np.random.default_rng(65)
+    mask = (rng.random((B, Sq, Sk)) < 0.3).astype(np.uint8)
+    mask[:, :, 0] = 0                                    # every row keeps a visible key
+    drop = (rng.random((B, N, Sq, Sk)) < 0.8).astype(np.uint8)
+    okw = dict(scale=D ** -0.5, attn_mask=mask, drop_mask=drop, keep_prob=0.8)
+    _check_all(q, k, v, dO, okw, _run(q, k, v, dO, scale=D ** -0.5, mask_kind=_capi.MASK_DENSE_U8, attn_mask=mask,
+                                      drop_mask=drop, keep_prob=0.8))
+
+
 @pytest.mark.parametrize("form", ["row_bias", "full_bias"])
 def test_alibi_forms(form):
     B, N, S, D = 1, 8, 1024, 128
