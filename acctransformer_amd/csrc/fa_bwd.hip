@@ -133,9 +133,18 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   TileDma<T, D, 64, NW> kdma, vdma;
   kdma.plan(a.k_ss);
   vdma.plan(a.v_ss);
+  // bias tiles of this wave's rows are staged through a wave-private LDS region one tile ahead
+  ACCT_LDS char* bias_lds = smem + 4 * TILEB + wave * (QG * 4096);
+  const bool bias_staged = BIAS && (a.Sk & 7) == 0 && (((uintptr_t)a.alibi & 15) | ((a.al_sb | a.al_sh | a.al_sq) & 7)) == 0;
+  auto stage_bias = [&](int jn) {
+#pragma unroll
+    for (int gq = 0; gq < QG; gq++)
+      bias_tile_dma<T>(alibip, a.al_sq, wq0 + 32 * gq, a.Sq, jn * 64, a.Sk, bias_lds + gq * 4096);
+  };
   if (j_lo <= j_hi) {
     tile_dma<T, D, 64, NW>(kp, a.k_ss, j_lo * 64, a.Sk, smem);
     tile_dma<T, D, 64, NW>(vp, a.v_ss, j_lo * 64, a.Sk, smem + TILEB);
+    if (BIAS && bias_staged && wq0 < a.Sq) stage_bias(j_lo);
     // A full wait the compiler can see: every load issued so far (Q, dO fragments included) is complete,
     // so it places no vmcnt wait inside the loop -- such a wait would also stall on the next tile's DMA.
     __builtin_amdgcn_s_waitcnt(0);
@@ -217,30 +226,61 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
                 ds[r] = p * (dp[gq][r] - dl[gq]);
               }
             } else {
+              // side inputs, in short passes over the 16 scores so that few values are live at a time
+              float x[16];
+#pragma unroll
+              for (int r = 0; r < 16; r++) x[r] = __builtin_fmaf(s[gq][r], a.scale_log2e, -lq[gq]);
+              if (BIAS) {
+                if (bias_staged) {
+                  typename E::V4 bv[4];
+#pragma unroll
+                  for (int r4 = 0; r4 < 4; r4++) bv[r4] = bias_tile_read<T>(bias_lds + gq * 4096, l32, 4 * c + r4, g);
+                  if (c == 1 && gq == QG - 1) {
+                    // the whole tile has been read: its LDS region can take the next tile, which has the
+                    // rest of this step to land (the end-of-step wait covers it)
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    if (j < j_hi) stage_bias(j + 1);
+                  }
+#pragma unroll
+                  for (int r = 0; r < 16; r++) x[r] = __builtin_fmaf((float)bv[r >> 2][r & 3], kLog2e, x[r]);
+                } else {
+#pragma unroll
+                  for (int r4 = 0; r4 < 4; r4++) {
+                    float bias[4];
+                    load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv0 + 32 * c + 8 * r4 + 4 * g, a.Sk, alibi_vec, bias);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) x[4 * r4 + e] = __builtin_fmaf(bias[e], kLog2e, x[4 * r4 + e]);
+                  }
+                }
+              }
+              if (apply_mask) {
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {
+                  const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
+                  uint32_t mbits;
+                  if (a.mask_kind == kMaskDense) mbits = load_u8x4(maskp + (int64_t)qrow_c * a.Sk, kv, a.Sk, mask_vec);
+                  else mbits = load_u8x4(maskp + (qrow_c & 127) * 128, kv & 127, 128, mask_vec);
+#pragma unroll
+                  for (int e = 0; e < 4; e++)
+                    if ((mbits >> (8 * e)) & 0xffu) x[4 * r4 + e] += kMaskFill * kLog2e;
+                }
+              }
+              {
+                // keys after the query (causal) or past Sk: P is exactly 0
+                int vis = a.Sk - 1 - kv0 - 32 * c - 4 * g;
+                if (causal) vis = min(vis, qrow - kv0 - 32 * c - 4 * g);
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                  if (8 * (r >> 2) + (r & 3) > vis) x[r] = -INFINITY;
+              }
               uint32_t dw = 0xffffffffu;                        // keep bits of this row: keys kv0 + 32c .. +31
               if (DROP) dw = a.droprow[((int64_t)bh * a.Sq + qrow_c) * a.droprow_w + 2 * j + c] >> (4 * g);
 #pragma unroll
-              for (int r4 = 0; r4 < 4; r4++) {
-                const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
-                float bias[4] = {0.f, 0.f, 0.f, 0.f};
-                uint32_t mbits = 0;
-                if (BIAS) load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
-                if (apply_mask) {
-                  if (a.mask_kind == kMaskDense) mbits = load_u8x4(maskp + (int64_t)qrow_c * a.Sk, kv, a.Sk, mask_vec);
-                  else mbits = load_u8x4(maskp + (qrow_c & 127) * 128, kv & 127, 128, mask_vec);
-                }
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                  const int r = 4 * r4 + e;
-                  float x = __builtin_fmaf(s[gq][r], a.scale_log2e, -lq[gq]);
-                  if (BIAS) x = __builtin_fmaf(bias[e], kLog2e, x);
-                  if (((mbits >> (8 * e)) & 0xffu) || (causal && kv + e > qrow)) x += kMaskFill * kLog2e;
-                  float p = fast_exp2(x);
-                  if (kv + e >= a.Sk) p = 0.f;
-                  float dpv = dp[gq][r];
-                  if (DROP) dpv = ((dw >> (8 * r4 + e)) & 1u) ? dpv * a.inv_keep : 0.f;
-                  ds[r] = p * (dpv - dl[gq]);
-                }
+              for (int r = 0; r < 16; r++) {
+                const float p = fast_exp2(x[r]);
+                float dpv = dp[gq][r];
+                if (DROP) dpv = ((dw >> (8 * (r >> 2) + (r & 3))) & 1u) ? dpv * a.inv_keep : 0.f;
+                ds[r] = p * (dpv - dl[gq]);
               }
             }
             dsf[gq][c][0] = pack8<T>(ds);
@@ -259,6 +299,8 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 #pragma unroll
               for (int gq = 0; gq < QG; gq++) acc[gq][db] = E::mfma(ktf, dsf[gq][c][hh], acc[gq][db]);
             }
+      } else if (BIAS && bias_staged && j < j_hi && wq0 < a.Sq) {
+        stage_bias(j + 1);                                  // nothing to read in this step: the region is free
       }
       dma_wait();
       __syncthreads();
@@ -669,7 +711,7 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
     constexpr int QG = 1, NW = 8;
     constexpr int BM = 32 * QG * NW;
     using CS = SwzCfg<D>;
-    constexpr size_t tiles = 4 * 64 * (size_t)CS::PITCH, stage = (size_t)NW * 32 * (CS::DB * 64 + 16);
+    constexpr size_t tiles = 4 * 64 * (size_t)CS::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0), stage = (size_t)NW * 32 * (CS::DB * 64 + 16);
     const size_t smem = tiles > stage ? tiles : stage;
     a.n_tiles = (a.Sq + BM - 1) / BM;
     const bool mask_q = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;

@@ -272,6 +272,12 @@ struct TileDma {
     asm volatile("" : "+v"(tid));
     const int lane = tid & 63, wave = tid >> 6;
     const T* tile = base + (int64_t)row0 * row_stride;
+    {
+      const uint64_t t = (uint64_t)(uintptr_t)tile;               // uniform: pinned in scalar registers
+      const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)t);
+      const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(t >> 32));
+      tile = (const T*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+    }
     const uint32_t dst0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)buf + (uint32_t)(wave * NIW * 1024));
     const uint32_t rs = (uint32_t)row_stride * (uint32_t)sizeof(T);
 #pragma unroll
@@ -285,7 +291,13 @@ struct TileDma {
   }
   // rows [row0, row0 + ROWS) must exist
   ACCT_DEV void issue(const T* base, int64_t row_stride, int row0, ACCT_LDS char* buf) const {
-    const T* tile = base + (int64_t)row0 * row_stride;            // uniform: lives in scalar registers
+    const T* tile = base + (int64_t)row0 * row_stride;            // uniform: must live in scalar registers
+    {
+      const uint64_t t = (uint64_t)(uintptr_t)tile;               // (pinned there: under register pressure the
+      const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)t);          // compiler may hold it in VGPRs)
+      const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(t >> 32));
+      tile = (const T*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+    }
     const uint32_t dst0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)buf) + lds0;
 #pragma unroll
     for (int i = 0; i < NIW; i++)
@@ -293,6 +305,32 @@ struct TileDma {
                    : "memory");
   }
 };
+
+// Wave-private staging of an additive-bias tile (32 query rows x 64 keys, 128 bytes per row) through LDS:
+// the lanes of the attention kernels own query rows, so direct loads would touch 32 different cache lines
+// per instruction; four 16-byte DMA instructions fetch whole rows instead.  The 16-byte chunk c of row r is
+// stored in slot c ^ (r & 7), which spreads the 8-byte reads of 8 consecutive rows over all banks.
+// Requires Sk % 8 == 0 and 16-byte aligned rows; rows past nrows repeat the last row, chunks past Sk repeat
+// the last chunk (their scores are masked anyway).
+template <typename T>
+ACCT_DEV void bias_tile_dma(const T* base, int64_t row_stride, int row0, int nrows, int kv0, int Sk, ACCT_LDS char* dst) {
+  int ln = threadIdx.x & 63;
+  asm volatile("" : "+v"(ln));
+  const int lcm = (Sk - kv0) / 8 - 1;              // last chunk of this tile that lies inside the row
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int r = 8 * i + (ln >> 3);
+    const int lc = min((ln & 7) ^ (r & 7), lcm);
+    const T* src = base + (int64_t)min(row0 + r, nrows - 1) * row_stride + kv0 + 8 * lc;
+    const uint32_t d = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(dst + i * 1024));
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(d) : "memory");
+  }
+}
+// the 4 bias values of row `row` (0..31) for keys 8*cc + 4*half .. +3 of the staged tile
+template <typename T>
+ACCT_DEV typename Elem<T>::V4 bias_tile_read(const ACCT_LDS char* tile, int row, int cc, int half) {
+  return *reinterpret_cast<const ACCT_LDS typename Elem<T>::V4*>(tile + row * 128 + ((cc ^ (row & 7)) << 4) + 8 * half);
+}
 
 // all of this wave's direct-to-LDS loads have landed
 ACCT_DEV void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }

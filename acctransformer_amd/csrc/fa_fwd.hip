@@ -100,9 +100,18 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   TileDma<T, D, 64, NW> kdma, vdma;
   kdma.plan(a.k_ss);
   vdma.plan(a.v_ss);
+  // bias tiles of this wave's rows are staged through a wave-private LDS region one tile ahead
+  ACCT_LDS char* bias_lds = smem + 4 * TILEB + wave * (QG * 4096);
+  const bool bias_staged = BIAS && (a.Sk & 7) == 0 && (((uintptr_t)a.alibi & 15) | ((a.al_sb | a.al_sh | a.al_sq) & 7)) == 0;
+  auto stage_bias = [&](int jn) {
+#pragma unroll
+    for (int gq = 0; gq < QG; gq++)
+      bias_tile_dma<T>(alibip, a.al_sq, wq0 + 32 * gq, a.Sq, jn * 64, a.Sk, bias_lds + gq * 4096);
+  };
   if (j_lo <= j_hi) {
     tile_dma<T, D, 64, NW>(kp, a.k_ss, j_lo * 64, a.Sk, smem);
     tile_dma<T, D, 64, NW>(vp, a.v_ss, j_lo * 64, a.Sk, smem + TILEB);
+    if (BIAS && bias_staged && wq0 < a.Sq) stage_bias(j_lo);
     // A full wait the compiler can see: every load issued so far (Q fragments included) is complete, so
     // it places no vmcnt wait inside the loop -- such a wait would also stall on the next tile's DMA.
     __builtin_amdgcn_s_waitcnt(0);
@@ -173,17 +182,38 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
           const int qrow = wq0 + 32 * gq + l32;
           const int qrow_c = min(qrow, a.Sq - 1);            // clamped for side-input addressing
           if (BIAS) {
+            if (bias_staged) {
+              typename E::V4 bv[2][4];
 #pragma unroll
-            for (int c = 0; c < 2; c++)
+              for (int c = 0; c < 2; c++)
 #pragma unroll
-              for (int r4 = 0; r4 < 4; r4++) {
-                const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
-                float bias[4];
-                load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                  s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale_log2e, bias[e] * kLog2e);
+                for (int r4 = 0; r4 < 4; r4++) bv[c][r4] = bias_tile_read<T>(bias_lds + gq * 4096, l32, 4 * c + r4, g);
+              if (gq == QG - 1) {
+                // the tile is in registers: its LDS region can take the next tile, which has the rest of
+                // this step to land (the end-of-step wait covers it)
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (j < j_hi) stage_bias(j + 1);
               }
+#pragma unroll
+              for (int c = 0; c < 2; c++)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++)
+#pragma unroll
+                  for (int e = 0; e < 4; e++)
+                    s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale_log2e, (float)bv[c][r4][e] * kLog2e);
+            } else {
+#pragma unroll
+              for (int c = 0; c < 2; c++)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {
+                  const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
+                  float bias[4];
+                  load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
+#pragma unroll
+                  for (int e = 0; e < 4; e++)
+                    s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale_log2e, bias[e] * kLog2e);
+                }
+            }
           }
           if (edge) {
             if (apply_mask) {
@@ -290,6 +320,8 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
 #pragma unroll
               for (int gq = 0; gq < QG; gq++) o[gq][db] = E::mfma(vf, pf[gq][c][hh], o[gq][db]);
             }
+      } else if (BIAS && bias_staged && j < j_hi && wq0 < a.Sq) {
+        stage_bias(j + 1);                                  // nothing to read in this step: the region is free
       }
       TR(4);
       dma_wait();
@@ -343,7 +375,7 @@ static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
   using C = SwzCfg<D>;
   constexpr int BM = 32 * QG * NW;
   a.n_tiles = (a.Sq + BM - 1) / BM;
-  constexpr size_t tiles = 4 * 64 * (size_t)C::PITCH, stage = (size_t)NW * 32 * (C::DB * 64 + 16);
+  constexpr size_t tiles = 4 * 64 * (size_t)C::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0), stage = (size_t)NW * 32 * (C::DB * 64 + 16);
   const size_t smem = tiles > stage ? tiles : stage;
   const bool mask_t = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;
   auto kern = mask_t ? fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, true> : fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, BIAS || DROP>;
