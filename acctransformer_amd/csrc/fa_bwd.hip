@@ -352,6 +352,10 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 #ifndef ACCT_PARK_HOT
 #define ACCT_PARK_HOT 4      // the variant without side inputs has registers for two more fragments
 #endif
+// stationary fragments parked in LDS per wave: the bias variants give one up for the bias tiles' LDS
+template <int D, bool BIAS, bool MASKT>
+constexpr int dkdv_park() { return D >= 128 ? (BIAS ? ACCT_PARK - 1 : (MASKT ? ACCT_PARK : ACCT_PARK_HOT)) : 0; }
+
 ACCT_DEV void dma4(const void* src, ACCT_LDS char* dst) {
   const uint32_t d = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst);
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(d) : "memory");
@@ -401,9 +405,11 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   // lane holds key row 32 gk + l32, d = 16t + 8g ..
   // The last PARK k-steps of the second key group live in a wave-private LDS slab instead of
   // registers (16 VGPRs at D = 128): that is what lets two waves share a SIMD without spilling.
-  constexpr int PARK = D >= 128 ? (MASKT ? ACCT_PARK : ACCT_PARK_HOT) : 0;
+  constexpr int PARK = dkdv_park<D, BIAS, MASKT>();
   V8 bf[2][C::KS];
   ACCT_LDS char* park = pexch + 8 * PXB + wave * (PARK * 1024) + lane * 16;
+  // bias tile (32 query rows x the pair's 64 keys) of the V-role wave, staged one chunk ahead by DMA
+  ACCT_LDS char* bias_lds = pexch + 8 * PXB + 8 * (PARK * 1024) + pair * 4096;
   {
     const T* src = krole ? vp : kp;
     const int64_t ss = krole ? a.v_ss : a.k_ss;
@@ -456,6 +462,10 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     }
   };
 
+  const bool bias_staged = BIAS && !krole && wk0 < a.Sk && (a.Sk & 7) == 0 &&
+                           (((uintptr_t)a.alibi & 15) | ((a.al_sb | a.al_sh | a.al_sq) & 7)) == 0;
+  auto stage_bias = [&](int cn) { bias_tile_dma<T, false>(alibip, a.al_sq, cn * 32, a.Sq, wk0, a.Sk, bias_lds); };
+
   // per-chunk predicates of this pair (chunk = 32 query rows; two per staged tile)
   auto classify = [&](int cidx, bool& act, bool& apply_mask, bool& edge) {
     const int qc0 = cidx * 32, qt0 = (cidx >> 1) * 64, qb = cidx >> 2;
@@ -475,6 +485,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 
   if (i_lo <= i_hi) {
     stage(i_lo, smem);
+    if (BIAS && bias_staged) stage_bias(2 * i_lo);
     // A full wait the compiler can see: the stationary fragments loaded above are complete, so it places
     // no vmcnt wait inside the loop -- such a wait would also stall on the next tile's DMA.
     __builtin_amdgcn_s_waitcnt(0);
@@ -557,7 +568,19 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
               // passes that each keep few values live: + bias/scale; - 10000/scale where the mask bit of
               // (row, key) is set; -inf where the key comes after the query (causal) or where the key
               // or the query row does not exist (the probability is exactly 0 either way).
-              if (BIAS) {
+              if (BIAS && bias_staged) {
+                const ACCT_LDS char* bl = bias_lds + g * 512 + l32 * 2;     // row 4g, key l32 of the staged tile
+#pragma unroll
+                for (int gk = 0; gk < 2; gk++)
+#pragma unroll
+                  for (int r = 0; r < 16; r++) {
+                    const T bv = *reinterpret_cast<const ACCT_LDS T*>(bl + (8 * (r >> 2) + (r & 3)) * 128 + gk * 64);
+                    t0[gk][r] += (float)bv * a.inv_scale;
+                    if ((r & 7) == 7) asm volatile("" ::: "memory");
+                  }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // tile consumed: stage the next chunk's
+                if (n < c_hi) stage_bias(n + 1);
+              } else if (BIAS) {
                 const int qlast = a.Sq - 1 - qc0;               // last valid row, relative to the chunk
                 const T* brow0 = alibip + (int64_t)qc0 * a.al_sq;
 #pragma unroll
@@ -657,6 +680,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 #pragma unroll
               for (int gk = 0; gk < 2; gk++) acc[gk][db] = E::mfma(af, bfr[gk][hh], acc[gk][db]);
             }
+        } else if (BIAS && bias_staged && n < c_hi) {
+          stage_bias(n + 1);                            // nothing to read in this step: the region is free
         }
       }
       TR(3);
@@ -725,7 +750,8 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
   if (stages & kStageDkDv) {
     using CS = SwzCfg<D>;
     constexpr size_t stageb = 2 * 64 * (size_t)CS::PITCH + 512;
-    constexpr size_t loopb = 2 * stageb + 8 * 4096 + 8 * (D >= 128 ? ACCT_PARK : 0) * 1024, epib = (size_t)8 * 32 * (CS::DB * 64 + 16);
+    constexpr size_t loopb = 2 * stageb + 8 * 4096 + 8 * (size_t)dkdv_park<D, BIAS, true>() * 1024 + (BIAS ? 4 * 4096 : 0),
+                     epib = (size_t)8 * 32 * (CS::DB * 64 + 16);
     const size_t smem2 = loopb > epib ? loopb : epib;
     a.n_tiles = (a.Sk + 255) / 256;
     const bool mask_t = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;

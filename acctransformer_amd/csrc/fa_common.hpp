@@ -312,7 +312,8 @@ struct TileDma {
 // stored in slot c ^ (r & 7), which spreads the 8-byte reads of 8 consecutive rows over all banks.
 // Requires Sk % 8 == 0 and 16-byte aligned rows; rows past nrows repeat the last row, chunks past Sk repeat
 // the last chunk (their scores are masked anyway).
-template <typename T>
+// SWZ = false stores the rows plainly (for readers that walk down a column).
+template <typename T, bool SWZ = true>
 ACCT_DEV void bias_tile_dma(const T* base, int64_t row_stride, int row0, int nrows, int kv0, int Sk, ACCT_LDS char* dst) {
   int ln = threadIdx.x & 63;
   asm volatile("" : "+v"(ln));
@@ -320,7 +321,7 @@ ACCT_DEV void bias_tile_dma(const T* base, int64_t row_stride, int row0, int nro
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int r = 8 * i + (ln >> 3);
-    const int lc = min((ln & 7) ^ (r & 7), lcm);
+    const int lc = min(SWZ ? (ln & 7) ^ (r & 7) : (ln & 7), lcm);
     const T* src = base + (int64_t)min(row0 + r, nrows - 1) * row_stride + kv0 + 8 * lc;
     const uint32_t d = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(dst + i * 1024));
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(d) : "memory");
