@@ -3,7 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 One step = one forward call and one backward call of the attention operator
-through the C ABI, on the workload BASELINE.json quotes its metric on:
+through the C ABI, on the workload the headline metric is quoted on:
 B=4, N=16, S=2048, D=128, fp16, causal attn_mask (uint8, 1 = masked),
 keep_prob = 1, upstream dO ~ N(0,1).  Inputs are synthetic and already resident
 in HBM.  Prints one JSON line: whole-job TFLOP/s by the FlashAttention-2 flop
