@@ -771,12 +771,15 @@ static hipError_t launch_bwd_d(const FaArgs& a, int stages, hipStream_t st) {
 #ifndef ACCT_DEV_BUILD
   if (bias) return drop ? launch_bwd_t<T, D, true, true>(a, stages, st) : launch_bwd_t<T, D, true, false>(a, stages, st);
   if (drop) return launch_bwd_t<T, D, false, true>(a, stages, st);
+#else
+  if (bias || drop) return hipErrorNotSupported;       // development build: plain variants only
 #endif
   return launch_bwd_t<T, D, false, false>(a, stages, st);
 }
 
 hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t st) {
 #ifdef ACCT_DEV_BUILD
+  if (dtype != 0 || D != 128) return hipErrorNotSupported;
   return launch_bwd_d<f16, 128>(a, stages, st);
 #else
   if (dtype == 0) {

@@ -393,6 +393,8 @@ static hipError_t launch_fwd_q(const FaArgs& a, hipStream_t st) {
 #ifndef ACCT_DEV_BUILD
   if (bias) return drop ? launch_fwd_t<T, D, QG, NW, true, true>(a, st) : launch_fwd_t<T, D, QG, NW, true, false>(a, st);
   if (drop) return launch_fwd_t<T, D, QG, NW, false, true>(a, st);
+#else
+  if (bias || drop) return hipErrorNotSupported;       // development build: plain variants only
 #endif
   return launch_fwd_t<T, D, QG, NW, false, false>(a, st);
 }
@@ -406,6 +408,7 @@ static hipError_t launch_fwd_d(const FaArgs& a, int variant, hipStream_t st) {
 
 hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st) {
 #ifdef ACCT_DEV_BUILD
+  if (dtype != 0 || D != 128) return hipErrorNotSupported;
   return launch_fwd_d<f16, 128>(a, qg, st);
 #else
   if (dtype == 0) {

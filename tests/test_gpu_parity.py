@@ -221,6 +221,25 @@ def test_ragged_dropout_with_random_mask(Sq, Sk):
                                       drop_mask=drop, keep_prob=0.8))
 
 
+@pytest.mark.parametrize("dtype, Sq, Sk, D", [(torch.float16, 333, 328, 128), (torch.float16, 200, 333, 128),
+                                              (torch.bfloat16, 300, 456, 128), (torch.float16, 260, 392, 80)])
+def test_all_side_inputs_ragged(dtype, Sq, Sk, D):
+    # bias + dense mask + dropout together, at lengths where the bias staging (needs Sk % 8 == 0, else the
+    # direct loads), the keep-bit packing and the mask bitmaps all have partial pieces
+    B, N = 2, 3
+    q, dO = (_gen((B, N, Sq, D), s, dtype) for s in (71, 74))
+    k, v = (_gen((B, N, Sk, D), s, dtype) for s in (72, 73))
+    rng = np.random.default_rng(75)
+    mask = (rng.random((B, Sq, Sk)) < 0.25).astype(np.uint8)
+    mask[:, :, 0] = 0
+    drop = (rng.random((B, N, Sq, Sk)) < 0.85).astype(np.uint8)
+    al = (0.05 * torch.randn((1, N, Sq, Sk), generator=torch.Generator().manual_seed(76))).to(dtype)
+    okw = dict(scale=D ** -0.5, attn_mask=mask, drop_mask=drop, keep_prob=0.85, alibi=al.float().numpy())
+    tol = dict(atol=2e-2, rtol=1e-2) if dtype == torch.bfloat16 else {}
+    _check_all(q, k, v, dO, okw, _run(q, k, v, dO, scale=D ** -0.5, mask_kind=_capi.MASK_DENSE_U8, attn_mask=mask,
+                                      drop_mask=drop, keep_prob=0.85, alibi=al), **tol)
+
+
 @pytest.mark.parametrize("form", ["row_bias", "full_bias"])
 def test_alibi_forms(form):
     B, N, S, D = 1, 8, 1024, 128
