@@ -80,6 +80,8 @@ def load():
     lib.acct_fa_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.acct_last_error.argtypes = []
     lib.acct_last_error.restype = ctypes.c_char_p
+    lib.acct_build_is_complete.argtypes = []
+    lib.acct_build_is_complete.restype = ctypes.c_int
     lib.acct_version.argtypes = []
     lib.acct_version.restype = ctypes.c_int
     _lib = lib

@@ -154,6 +154,7 @@ extern "C" {
 
 const char* acct_last_error(void) { return g_err; }
 int acct_version(void) { return ACCT_FA_VERSION; }
+int acct_build_is_complete(void) { return acct::launch_variants_complete() ? 1 : 0; }
 
 size_t acct_fa_fwd_workspace_bytes(const acct_fa_params* p) {
   if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0 || p->Sk <= 0) return 0;

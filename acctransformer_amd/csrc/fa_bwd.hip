@@ -777,6 +777,13 @@ static hipError_t launch_bwd_d(const FaArgs& a, int stages, hipStream_t st) {
   return launch_bwd_t<T, D, false, false>(a, stages, st);
 }
 
+bool fwd_variants_complete();
+#ifdef ACCT_DEV_BUILD
+bool launch_variants_complete() { return false; }
+#else
+bool launch_variants_complete() { return fwd_variants_complete(); }
+#endif
+
 hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t st) {
 #ifdef ACCT_DEV_BUILD
   if (dtype != 0 || D != 128) return hipErrorNotSupported;

@@ -406,6 +406,12 @@ static hipError_t launch_fwd_d(const FaArgs& a, int variant, hipStream_t st) {
   return variant == 2 ? launch_fwd_q<T, D, 2, 4>(a, st) : launch_fwd_q<T, D, 1, 4>(a, st);
 }
 
+#ifdef ACCT_DEV_BUILD
+bool fwd_variants_complete() { return false; }
+#else
+bool fwd_variants_complete() { return true; }
+#endif
+
 hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st) {
 #ifdef ACCT_DEV_BUILD
   if (dtype != 0 || D != 128) return hipErrorNotSupported;

@@ -12,6 +12,9 @@ hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st)
 enum : int { kStageDq = 1, kStageDkDv = 2 };
 hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t st);
 
+// false when the kernel translation units were compiled with a reduced variant set (ACCT_DEV_BUILD)
+bool launch_variants_complete();
+
 // classify the 128x128 blocks of a dense uint8 mask into clean / apply / skip
 hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, int MB, hipStream_t st);
 // pack the dropout mask into keep bits by query row [B*N, Sq, droprow_w] and / or by key column [B*N, Tr, Sk, 4]

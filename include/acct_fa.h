@@ -128,6 +128,11 @@ const char* acct_last_error(void);
 /* ACCT_FA_VERSION of the loaded library. */
 int acct_version(void);
 
+/* 1 when the library contains every element type, head dim and side-input variant; 0 for a development build
+ * that was compiled with a reduced variant set (such a build refuses the calls it cannot serve with
+ * ACCT_E_LAUNCH).  No counterpart in the reference: a guard for packaging and tests. */
+int acct_build_is_complete(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -33,6 +33,8 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
     m = re.search(r"#define ACCT_FA_VERSION (\d+)", _header())
     assert lib.acct_version() == int(m.group(1))
+    # the in-tree library must be the complete build, not a reduced development build
+    assert lib.acct_build_is_complete() == 1
 
 
 def test_struct_mirror_matches_header_field_order():
