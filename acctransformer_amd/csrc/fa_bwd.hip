@@ -76,6 +76,18 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   const bool causal = a.mask_kind == kMaskCausal;
   if (causal) j_hi = min(j_hi, (q_end - 1) / 64);
   if (a.row_prefix) j_hi = min(j_hi, (((q_end - 1) / a.row_prefix + 1) * a.row_prefix - 1) / 64);
+  if (MASKT && a.mask_kind == kMaskDense) {
+    // tiles at either end whose 128x128 blocks are wholly masked for every row block of this workgroup are
+    // not streamed at all (key padding: the padded tail of every sequence)
+    const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc;
+    auto dead = [&](int j) {
+      for (int qb = qb_lo; qb <= qb_hi; qb++)
+        if (fl[(int64_t)qb * a.Tc + (j >> 1)] != kBlkSkip) return false;
+      return true;
+    };
+    while (j_lo <= j_hi && dead(j_lo)) j_lo++;
+    while (j_lo <= j_hi && dead(j_hi)) j_hi--;
+  }
   const int wqb = wq0 / 128;
   const int wkv_limit = a.row_prefix ? (wq0 / a.row_prefix + 1) * a.row_prefix : 0x7fffffff;
 
@@ -400,6 +412,18 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   int i_lo = qb_lo * 2, i_hi = min(qb_hi * 2 + 1, (a.Sq - 1) / 64);
   const bool causal = a.mask_kind == kMaskCausal;
   if (causal) i_lo = max(i_lo, k0 / 64);            // query tiles wholly above the diagonal contribute 0
+  if (MASKT && a.mask_kind == kMaskDense) {
+    // query tiles at either end whose blocks are wholly masked for every key block of this workgroup are
+    // not streamed at all (key padding: a workgroup of padded keys has nothing to do)
+    const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc;
+    auto dead = [&](int i) {
+      for (int kb = kb_lo; kb <= kb_hi; kb++)
+        if (fl[(int64_t)(i >> 1) * a.Tc + kb] != kBlkSkip) return false;
+      return true;
+    };
+    while (i_lo <= i_hi && dead(i_lo)) i_lo++;
+    while (i_lo <= i_hi && dead(i_hi)) i_hi--;
+  }
   const int wkb = wk0 / 128;
 
   // stationary B operands: K fragments (V role) or V fragments (K role) of the pair's 64 key rows;

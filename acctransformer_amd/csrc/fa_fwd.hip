@@ -51,6 +51,18 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   const bool causal = a.mask_kind == kMaskCausal;
   if (causal) j_hi = min(j_hi, (q_end - 1) / 64);
   if (a.row_prefix) j_hi = min(j_hi, (((q_end - 1) / a.row_prefix + 1) * a.row_prefix - 1) / 64);
+  if (MASKT && a.mask_kind == kMaskDense) {
+    // tiles at either end whose 128x128 blocks are wholly masked for every row block of this workgroup are
+    // not streamed at all (key padding: the padded tail of every sequence)
+    const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc;
+    auto dead = [&](int j) {
+      for (int qb = qb_lo; qb <= qb_hi; qb++)
+        if (fl[(int64_t)qb * a.Tc + (j >> 1)] != kBlkSkip) return false;
+      return true;
+    };
+    while (j_lo <= j_hi && dead(j_lo)) j_lo++;
+    while (j_lo <= j_hi && dead(j_hi)) j_hi--;
+  }
   const int wqb = wq0 / 128;                                // 128-block of this wave's rows
   const int wkv_limit = a.row_prefix ? (wq0 / a.row_prefix + 1) * a.row_prefix : 0x7fffffff;   // keys past it are absent
 
