@@ -121,12 +121,12 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   // per-lane LDS offsets (tile-invariant)
   int koff[C::KS];
 #pragma unroll
-  for (int t = 0; t < C::KS; t++) koff[t] = l32 * C::PITCH + swz_off(2 * t + g, swz3(l32));
+  for (int t = 0; t < C::KS; t++) koff[t] = l32 * C::PITCH + swz_off(2 * t + g, C::swz(l32));
   const int trow = 4 * g + ((lane & 15) >> 2);
   const int tchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
   int toff[C::DB];
 #pragma unroll
-  for (int db = 0; db < C::DB; db++) toff[db] = trow * C::PITCH + swz_off(4 * db + tchunk, swz3(trow)) + 8 * (lane & 1);
+  for (int db = 0; db < C::DB; db++) toff[db] = trow * C::PITCH + swz_off(4 * db + tchunk, C::swz(trow)) + 8 * (lane & 1);
 
   f32x16 acc[QG][C::DB];
 #pragma unroll
@@ -308,7 +308,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 #pragma unroll
             for (int db = 0; db < C::DB; db++) {
               const ACCT_LDS char* kaddr = kbuf + toff[db] + (32 * c + 16 * hh) * C::PITCH;
-              const V8 ktf = join_tr<T>(lds_read_tr(kaddr), lds_read_tr(kaddr + 8 * C::PITCH));
+              const V8 ktf = join_tr<T>(lds_read_tr(kaddr), lds_read_tr(kaddr + C::tr_hi(db)));
 #pragma unroll
               for (int gq = 0; gq < QG; gq++) acc[gq][db] = E::mfma(ktf, dsf[gq][c][hh], acc[gq][db]);
             }
@@ -458,7 +458,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
       for (int r = 0; r < 16; r++) acc[gk][db][r] = 0.f;
 
   // per-lane LDS offsets (tile-invariant)
-#define FOFF(t) (foff4[(t) & 3] + ((t) >> 2) * 128)
+#define FOFF(t) (foff4[(t) & 3] ^ (((t) >> 2) * 128))
 #define TOFF(db) (toff2[(db) & 1] + ((db) >> 1) * 128)
 #ifdef ACCT_NO_EDGE
 #define EDGE_PATH false
@@ -535,19 +535,19 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
         if (act) {
           const int c = cidx & 1, qc0 = cidx * 32;
           // Per-lane LDS offsets are re-derived in every step (a handful of VALU ops) rather than
-          // kept in registers.  The swizzle only touches the low three bits of the chunk index, so
-          // chunk c + 8 sits 128 bytes after chunk c: four (two) base offsets plus immediates cover
-          // all fragments of a row.
+          // kept in registers.  Chunk c + 8 of a row sits in slot (c ^ swz) ^ 8: the row-major
+          // fragments of the upper half of the head dim are one XOR away from the lower four, and the
+          // transposed ones (row % 16 < 8, swizzle bit 3 clear) 128 bytes after them.
           int ln = lane;
           asm volatile("" : "+v"(ln));
           int foff4[4];                               // row-major fragment of k-step t: row l32, chunk 2t + g
 #pragma unroll
-          for (int t = 0; t < 4; t++) foff4[t] = (ln & 31) * C::PITCH + swz_off(2 * t + (ln >> 5), swz3(ln & 31));
+          for (int t = 0; t < 4; t++) foff4[t] = (ln & 31) * C::PITCH + swz_off(2 * t + (ln >> 5), C::swz(ln & 31));
           const int trow = 4 * (ln >> 5) + ((ln & 15) >> 2);
           const int tchunk = 2 * ((ln >> 4) & 1) + ((ln & 3) >> 1);
           int toff2[2];                               // transposed fragment of d block db
 #pragma unroll
-          for (int db = 0; db < 2; db++) toff2[db] = trow * C::PITCH + swz_off(4 * db + tchunk, swz3(trow)) + 8 * (ln & 1);
+          for (int db = 0; db < 2; db++) toff2[db] = trow * C::PITCH + swz_off(4 * db + tchunk, C::swz(trow)) + 8 * (ln & 1);
           ACCT_LDS char* qbuf = smem + (((cidx >> 1) - i_lo) & 1) * STAGEB;
           ACCT_LDS char* dobuf = qbuf + TILEB;
           const ACCT_LDS float* lbuf = (const ACCT_LDS float*)(qbuf + 2 * TILEB);
@@ -701,7 +701,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 #pragma unroll
             for (int db = 0; db < C::DB; db++) {
               const ACCT_LDS char* ta = tb + TOFF(db) + 16 * hh * C::PITCH;
-              const V8 af = join_tr<T>(lds_read_tr(ta), lds_read_tr(ta + 8 * C::PITCH));
+              const V8 af = join_tr<T>(lds_read_tr(ta), lds_read_tr(ta + C::tr_hi(db)));
 #pragma unroll
               for (int gk = 0; gk < 2; gk++) acc[gk][db] = E::mfma(af, bfr[gk][hh], acc[gk][db]);
             }

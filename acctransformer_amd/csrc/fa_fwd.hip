@@ -79,12 +79,12 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   // ---- per-lane LDS offsets (tile-invariant) ----
   int koff[C::KS];                                          // K fragment of k-step t: row l32, chunk 2t + g
 #pragma unroll
-  for (int t = 0; t < C::KS; t++) koff[t] = l32 * C::PITCH + swz_off(2 * t + g, swz3(l32));
+  for (int t = 0; t < C::KS; t++) koff[t] = l32 * C::PITCH + swz_off(2 * t + g, C::swz(l32));
   const int trow = 4 * g + ((lane & 15) >> 2);              // transposed reads: row within an 8-row group
   const int tchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
   int voff[C::DB];                                          // V^T fragment of d block db
 #pragma unroll
-  for (int db = 0; db < C::DB; db++) voff[db] = trow * C::PITCH + swz_off(4 * db + tchunk, swz3(trow)) + 8 * (lane & 1);
+  for (int db = 0; db < C::DB; db++) voff[db] = trow * C::PITCH + swz_off(4 * db + tchunk, C::swz(trow)) + 8 * (lane & 1);
 
   f32x16 o[QG][C::DB];
   float m[QG], lsum[QG];
@@ -329,7 +329,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
 #pragma unroll
             for (int db = 0; db < C::DB; db++) {
               const ACCT_LDS char* vaddr = vbuf + voff[db] + (32 * c + 16 * hh) * C::PITCH;
-              const V8 vf = join_tr<T>(lds_read_tr(vaddr), lds_read_tr(vaddr + 8 * C::PITCH));
+              const V8 vf = join_tr<T>(lds_read_tr(vaddr), lds_read_tr(vaddr + C::tr_hi(db)));
 #pragma unroll
               for (int gq = 0; gq < QG; gq++) o[gq][db] = E::mfma(vf, pf[gq][c][hh], o[gq][db]);
             }
