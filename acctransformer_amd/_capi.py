@@ -39,6 +39,7 @@ class AcctFaParams(ctypes.Structure):
         ("v_stride", ctypes.c_int64 * 3), ("o_stride", ctypes.c_int64 * 3),
         ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
         ("attn_mask", ctypes.c_void_p), ("drop_mask", ctypes.c_void_p), ("alibi", ctypes.c_void_p),
+        ("drop_seed", ctypes.c_uint64), ("drop_offset", ctypes.c_uint32), ("drop_philox", ctypes.c_int32),
     ]
 
 
@@ -105,11 +106,14 @@ def _bhs_strides(t):
 
 
 def make_params(q, k, v, *, scale, keep_prob=1.0, prev_block_num=BLOCK_UNBOUNDED, next_block_num=BLOCK_UNBOUNDED,
-                mask_kind=MASK_NONE, attn_mask=None, drop_mask=None, alibi=None, o_like=None, row_block_prefix=0):
+                mask_kind=MASK_NONE, attn_mask=None, drop_mask=None, alibi=None, o_like=None, row_block_prefix=0,
+                drop_seed=None, drop_offset=0):
     """Describe one attention problem.  q [B,N,Sq,D]; k,v [B,N,Sk,D] (any
     batch/head/row strides, unit stride along D); attn_mask uint8 [1|B,Sq,Sk]
     (DENSE) or [128,128] (TILE); drop_mask uint8 [B,N,Sq,Sk]; alibi in q's
-    dtype, broadcastable to [B,N,Sq,Sk]."""
+    dtype, broadcastable to [B,N,Sq,Sk].  With drop_seed (and no drop_mask) and
+    keep_prob < 1 the library draws the keep mask itself from
+    (drop_seed, drop_offset), identically in forward and backward."""
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be 4-D [B,N,S,D]")
     B, N, Sq, D = q.shape
@@ -152,6 +156,12 @@ def make_params(q, k, v, *, scale, keep_prob=1.0, prev_block_num=BLOCK_UNBOUNDED
             raise TypeError(f"drop_mask must be contiguous uint8 [{B},{N},{Sq},{Sk}]")
         p.drop_mask = drop_mask.data_ptr()
         keep.append(drop_mask)
+    if drop_seed is not None:
+        if drop_mask is not None:
+            raise ValueError("give either drop_mask or drop_seed, not both")
+        p.drop_seed = int(drop_seed) & 0xFFFFFFFFFFFFFFFF
+        p.drop_offset = int(drop_offset) & 0xFFFFFFFF
+        p.drop_philox = 1
     if alibi is not None:
         if alibi.dtype != q.dtype or alibi.dim() != 4 or alibi.shape[3] != Sk or alibi.stride(3) != 1:
             raise TypeError("alibi must be 4-D in q's dtype with a contiguous last dim of Sk")

@@ -49,6 +49,14 @@ size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 bool strides_zero(const int64_t s[3]) { return s[0] == 0 && s[1] == 0 && s[2] == 0; }
 
+// counter-based dropout is on: the keep mask comes from (drop_seed, drop_offset), not from a tensor
+bool philox_on(const acct_fa_params* p) { return p->drop_philox != 0 && !p->drop_mask && p->keep_prob < 1.f; }
+bool dropout_on(const acct_fa_params* p) { return p->drop_mask != nullptr || philox_on(p); }
+uint32_t philox_threshold(float keep_prob) {
+  long t = lroundf(256.f * keep_prob);
+  return (uint32_t)(t < 1 ? 1 : t > 256 ? 256 : t);
+}
+
 // Checks that need no device: used by the entry points and by the workspace queries.
 int validate(const acct_fa_params* p) {
   if (!p) return fail(ACCT_E_NULLPTR, "params is NULL");
@@ -109,6 +117,13 @@ acct::FaArgs make_args(const acct_fa_params* p) {
   a.scale = p->scale;
   a.scale_log2e = p->scale * acct::kLog2e;
   a.inv_keep = 1.0f / p->keep_prob;
+  if (philox_on(p)) {
+    a.philox_k0 = (uint32_t)p->drop_seed;
+    a.philox_k1 = (uint32_t)(p->drop_seed >> 32);
+    a.philox_offset = p->drop_offset;
+    a.philox_thr = philox_threshold(p->keep_prob);
+    a.inv_keep = 256.0f / (float)a.philox_thr;          // the reciprocal of the keep probability actually used
+  }
   a.inv_scale = 1.0f / p->scale;
   a.mask_add_raw = acct::kMaskFill / p->scale;
   a.prev_blk = p->prev_block_num > ACCT_BLOCK_UNBOUNDED ? ACCT_BLOCK_UNBOUNDED : p->prev_block_num;
@@ -135,11 +150,11 @@ size_t colbit_bytes(const acct_fa_params* p) {
 // keep bits of the dropout mask: by query row (forward, dQ) and by key column (dK/dV)
 size_t droprow_words(const acct_fa_params* p) { return 2 * (size_t)((p->Sk + 63) / 64); }   // 32-bit words per row
 size_t droprow_bytes(const acct_fa_params* p) {
-  if (!p->drop_mask) return 0;
+  if (!dropout_on(p)) return 0;
   return align_up((size_t)p->B * p->N * p->Sq * droprow_words(p) * 4, 256);
 }
 size_t dropcol_bytes(const acct_fa_params* p) {
-  if (!p->drop_mask) return 0;
+  if (!dropout_on(p)) return 0;
   return align_up((size_t)p->B * p->N * (size_t)((p->Sq + 127) / 128) * (size_t)p->Sk * 16, 256);
 }
 
@@ -173,7 +188,7 @@ int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, s
   if (rc) return rc;
   if (!O || !LSE) return fail(ACCT_E_NULLPTR, "O and LSE must be non-NULL");
   if ((uintptr_t)O & 7) return fail(ACCT_E_SHAPE, "O must be 8-byte aligned");
-  if (p->keep_prob < 1.f && !p->drop_mask) return fail(ACCT_E_NULLPTR, "keep_prob < 1 needs a drop_mask");
+  if (p->keep_prob < 1.f && !dropout_on(p)) return fail(ACCT_E_NULLPTR, "keep_prob < 1 needs a drop_mask or drop_philox");
   const size_t need = acct_fa_fwd_workspace_bytes(p);
   if (need && (!workspace || workspace_bytes < need))
     return fail(ACCT_E_WORKSPACE, "forward workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
@@ -188,11 +203,11 @@ int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, s
     hipError_t e = acct::launch_mask_blocks(a, (uint8_t*)workspace, p->mask_stride_b ? p->B : 1, st);
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
   }
-  if (p->drop_mask) {
+  if (dropout_on(p)) {
     uint32_t* rows = (uint32_t*)((char*)workspace + flag_bytes(p));
     a.droprow = rows;
     a.droprow_w = (int)droprow_words(p);
-    hipError_t e = acct::launch_drop_bits(a, rows, nullptr, st);
+    hipError_t e = philox_on(p) ? acct::launch_drop_philox(a, rows, nullptr, st) : acct::launch_drop_bits(a, rows, nullptr, st);
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "dropout bitmap kernel: %s", hipGetErrorString(e));
   }
   // 8 waves x 32 query rows (two waves per SIMD overlap MFMA and softmax work) once that still
@@ -214,7 +229,7 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
     return fail(ACCT_E_NULLPTR, "O, dO, LSE and the requested gradients must be non-NULL");
   if (((uintptr_t)O | (uintptr_t)dO | (uintptr_t)dQ | (uintptr_t)dK | (uintptr_t)dV) & 15)
     return fail(ACCT_E_SHAPE, "O, dO, dQ, dK and dV must be 16-byte aligned");
-  if (p->keep_prob < 1.f && !p->drop_mask) return fail(ACCT_E_NULLPTR, "keep_prob < 1 needs a drop_mask");
+  if (p->keep_prob < 1.f && !dropout_on(p)) return fail(ACCT_E_NULLPTR, "keep_prob < 1 needs a drop_mask or drop_philox");
   const size_t need = acct_fa_bwd_workspace_bytes(p);
   if (!workspace || workspace_bytes < need)
     return fail(ACCT_E_WORKSPACE, "backward workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
@@ -244,14 +259,15 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
     hipError_t e = acct::launch_mask_colbits(a, flags, cbits, p->mask_stride_b ? p->B : 1, st);
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask bitmap kernel: %s", hipGetErrorString(e));
   }
-  if (p->drop_mask) {
+  if (dropout_on(p)) {
     char* base = (char*)workspace + 2 * stat_bytes + flag_bytes(p) + colbit_bytes(p);
     uint32_t* rows = (uint32_t*)base;
     uint32_t* cols = (uint32_t*)(base + droprow_bytes(p));
     a.droprow = rows;
     a.dropcol = cols;
     a.droprow_w = (int)droprow_words(p);
-    hipError_t e = acct::launch_drop_bits(a, want_dq ? rows : nullptr, want_dkdv ? cols : nullptr, st);
+    hipError_t e = philox_on(p) ? acct::launch_drop_philox(a, want_dq ? rows : nullptr, want_dkdv ? cols : nullptr, st)
+                                : acct::launch_drop_bits(a, want_dq ? rows : nullptr, want_dkdv ? cols : nullptr, st);
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "dropout bitmap kernel: %s", hipGetErrorString(e));
   }
   hipError_t e = acct::launch_bwd(a, p->dtype, p->D, stages, st);

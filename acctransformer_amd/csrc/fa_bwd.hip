@@ -791,7 +791,7 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
 
 template <typename T, int D>
 static hipError_t launch_bwd_d(const FaArgs& a, int stages, hipStream_t st) {
-  const bool bias = a.alibi != nullptr, drop = a.drop != nullptr;
+  const bool bias = a.alibi != nullptr, drop = a.droprow != nullptr || a.dropcol != nullptr;
 #ifndef ACCT_DEV_BUILD
   if (bias) return drop ? launch_bwd_t<T, D, true, true>(a, stages, st) : launch_bwd_t<T, D, true, false>(a, stages, st);
   if (drop) return launch_bwd_t<T, D, false, true>(a, stages, st);

@@ -83,6 +83,23 @@ ACCT_DEV float pair_sum(float x) {
 
 ACCT_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11): ten rounds of
+// two 32x32->64 multiplies; the key is bumped by the Weyl constants after every round.
+ACCT_DEV void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1, uint32_t (&out)[4]) {
+#pragma unroll
+  for (int r = 0; r < 10; r++) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c1 = (uint32_t)p1;
+    c3 = (uint32_t)p0;
+    c0 = n0;
+    c2 = n2;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
 // ---- kernel arguments --------------------------------------------------------
 struct FaArgs {
   const void* q; const void* k; const void* v;
@@ -110,6 +127,8 @@ struct FaArgs {
   int row_prefix;                      // >0: row i sees keys j < (i/row_prefix + 1)*row_prefix only (multiple of 128)
   int n_tiles;                         // tiles along the owner dimension
   int droprow_w;                       // 32-bit words per row of droprow: 2 * ceil(Sk / 64)
+  uint32_t philox_k0, philox_k1;       // counter-based dropout: key, call offset and keep threshold (byte < thr keeps)
+  uint32_t philox_offset, philox_thr;
 };
 
 enum : int { kMaskNone = 0, kMaskDense = 1, kMaskTile = 3, kMaskCausal = 4 };

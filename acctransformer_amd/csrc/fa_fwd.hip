@@ -401,7 +401,7 @@ static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
 
 template <typename T, int D, int QG, int NW>
 static hipError_t launch_fwd_q(const FaArgs& a, hipStream_t st) {
-  const bool bias = a.alibi != nullptr, drop = a.drop != nullptr;
+  const bool bias = a.alibi != nullptr, drop = a.droprow != nullptr || a.dropcol != nullptr;
 #ifndef ACCT_DEV_BUILD
   if (bias) return drop ? launch_fwd_t<T, D, QG, NW, true, true>(a, st) : launch_fwd_t<T, D, QG, NW, true, false>(a, st);
   if (drop) return launch_fwd_t<T, D, QG, NW, false, true>(a, st);

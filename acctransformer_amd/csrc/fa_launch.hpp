@@ -5,7 +5,7 @@
 namespace acct {
 
 // forward: qg = query groups of 32 rows per wave (1 or 2); the bias / dropout
-// variants are picked from a.alibi / a.drop
+// variants are picked from a.alibi / a.droprow
 hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st);
 
 // backward: delta pre-pass, dK/dV kernel (kv-tile owner) and dQ kernel (q-tile owner)
@@ -19,6 +19,8 @@ bool launch_variants_complete();
 hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, int MB, hipStream_t st);
 // pack the dropout mask into keep bits by query row [B*N, Sq, droprow_w] and / or by key column [B*N, Tr, Sk, 4]
 hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st);
+// the same two bitmaps generated from (a.philox_k0, a.philox_k1, a.philox_offset, a.philox_thr) instead of read from a mask
+hipError_t launch_drop_philox(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st);
 // pack the 'apply' blocks of a dense mask into per-key-column bitmaps [MB, Tr, Sk, 4 x u32]
 hipError_t launch_mask_colbits(const FaArgs& a, const uint8_t* flags, uint32_t* out, int MB, hipStream_t st);
 

@@ -216,6 +216,61 @@ __global__ void __launch_bounds__(64) fa_drop_bits_kernel(const FaArgs a, uint32
   }
 }
 
+// The same bitmaps for counter-based dropout: nothing is read, the keep decisions come from Philox4x32-10.
+// One call yields the 16 bytes of one (query row, 32-key group M, half g): keys 32M + 8u + 4g + e for
+// u = 0..3, e = 0..3 -- the keys one lane of the attention kernels owns in a 32-key group, so a kernel
+// could also draw them in place.  One wave per (batch*head, 128 query rows, 1024 keys); lane 2L + g owns
+// (M = 32*span + L, g), the lane pair forms the 32-bit row word of group M.
+__global__ void __launch_bounds__(64) fa_drop_philox_kernel(const FaArgs a, uint32_t* rowbits, uint32_t* colbits) {
+  const int nspan = (a.Sk + 1023) / 1024;
+  const int span = blockIdx.x % nspan, qb = (blockIdx.x / nspan) % a.Tr, bh = blockIdx.x / (nspan * a.Tr);
+  const int lane = threadIdx.x, g = lane & 1;
+  const int grp = 32 * span + (lane >> 1);              // 32-key group = word index within the row
+  const bool writer = rowbits && g == 0 && grp < a.droprow_w;
+  uint32_t* rowout = rowbits + ((int64_t)bh * a.Sq + qb * 128) * a.droprow_w + grp;
+  const int nrow = min(128, a.Sq - qb * 128);
+  uint32_t cw[16][4];                                   // per key: four words of 32 rows, most significant bit first
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+#pragma unroll
+    for (int t = 0; t < 16; t++) cw[t][i] = 0u;
+#pragma unroll 2
+    for (int r = 0; r < 32; r++) {
+      const int rr = 32 * i + r;
+      uint32_t v[4];
+      philox4x32_10((uint32_t)(qb * 128 + rr), (uint32_t)(2 * grp + g), (uint32_t)bh, a.philox_offset, a.philox_k0, a.philox_k1, v);
+      uint32_t bits = 0;
+#pragma unroll
+      for (int t = 0; t < 16; t++) {                    // t = 4u + e
+        const uint32_t keep = ((v[t >> 2] >> (8 * (t & 3))) & 0xffu) < a.philox_thr ? 1u : 0u;
+        bits |= keep << (8 * (t >> 2) + (t & 3));
+        cw[t][i] = (cw[t][i] << 1) | (rr < nrow ? keep : 0u);
+      }
+      uint32_t x = bits << (4 * g);
+      x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xf, 0xf, true);    // lane ^ 1
+      if (writer && rr < nrow) *rowout = x;
+      rowout += a.droprow_w;
+    }
+  }
+  if (colbits) {
+#pragma unroll
+    for (int t = 0; t < 16; t++) {
+      const int key = 32 * grp + 8 * (t >> 2) + 4 * g + (t & 3);
+      if (key < a.Sk) {
+        u32x4 v = {__builtin_bitreverse32(cw[t][0]), __builtin_bitreverse32(cw[t][1]), __builtin_bitreverse32(cw[t][2]),
+                   __builtin_bitreverse32(cw[t][3])};
+        *reinterpret_cast<u32x4*>(colbits + (((int64_t)bh * a.Tr + qb) * a.Sk + key) * 4) = v;
+      }
+    }
+  }
+}
+
+hipError_t launch_drop_philox(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st) {
+  const long long nblk = (long long)a.B * a.N * a.Tr * ((a.Sk + 1023) / 1024);
+  hipLaunchKernelGGL(fa_drop_philox_kernel, dim3((unsigned)nblk), dim3(64), 0, st, a, rowbits, colbits);
+  return hipGetLastError();
+}
+
 hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st) {
   const long long nblk = (long long)a.B * a.N * a.Tr * ((a.Sk + 1023) / 1024);
   hipLaunchKernelGGL(fa_drop_bits_kernel, dim3((unsigned)nblk), dim3(64), 0, st, a, rowbits, colbits);

@@ -7,12 +7,16 @@ by fp16(head_dim ** -0.25) before the op (`:117,188-189`); here the product of
 those two factors is handed to the kernel as `scale`, which applies it to
 q k^T in fp32 -- two elementwise passes over q and k disappear and the scores
 carry one rounding less.  Dropout: the reference materialises an fp16
-{0, 1/keep_prob} mask with DropoutGenMask/DropoutDoMask (`:198-203`); here a
-uint8 Bernoulli(keep_prob) mask is drawn with torch's generator and the
-1/keep_prob factor is applied inside the kernel.
+{0, 1/keep_prob} mask with DropoutGenMask/DropoutDoMask (`:198-203`); here no
+mask tensor exists: every training call hands the op a fresh (seed, offset)
+pair and the library draws the keep decisions itself (Philox4x32-10), the same
+in forward and backward, and applies the 1/keep_prob factor inside the kernel.
+The seed follows torch's global seed, so `torch.manual_seed` makes a run
+repeatable.
 """
 from __future__ import annotations
 
+import itertools
 import math
 
 import torch
@@ -21,6 +25,7 @@ from acctransformer_amd.flash_attention.ops.flash_attention.flash_attention_impl
 
 __all__ = ['FlashAttention']
 HEAD_DIM_MAX_LIMIT = 256
+_layer_ids = itertools.count(1)
 
 
 class FlashAttention(torch.nn.Module):
@@ -58,6 +63,8 @@ class FlashAttention(torch.nn.Module):
         self.alibi = alibi
         self.dp, self.mp = dp, mp
         self.in_strategy = None
+        self._layer_id = next(_layer_ids)             # separates the dropout streams of different layers
+        self._calls = 0                               # one fresh mask per training call
         self.flash_attention = get_flash_attention(
             prev_block_num=prev_block_num,
             next_block_num=next_block_num,
@@ -86,7 +93,9 @@ class FlashAttention(torch.nn.Module):
                 "the head_num of query, key and value must be the same, "
                 "If different head_num are used, users need to change themselves to be same by tile.")
         if self.enable_dropout and self.training:
-            drop_mask = (torch.rand((bsz, head_num, seq_len, k.shape[2]), device=q.device) < self.keep_prob).to(torch.uint8)
+            seed = (torch.initial_seed() ^ (self._layer_id * 0x9E3779B97F4A7C15)) & 0xFFFFFFFFFFFFFFFF
+            drop_mask = (seed, self._calls & 0xFFFFFFFF)
+            self._calls += 1
         else:
             drop_mask = None
         o, _ = self.flash_attention(q, k, v, attn_mask, drop_mask, alibi_mask)

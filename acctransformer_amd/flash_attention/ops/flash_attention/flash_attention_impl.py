@@ -17,6 +17,10 @@ Differences from the reference that a caller can see:
     as "nonzero = masked" (the reference multiplies its value by -10000, and
     only ever feeds 0/1).  A floating dropout_mask is the reference's
     {0, 1/keep_prob} form; a uint8/bool one is {0,1} with `keep_prob` given.
+  * `dropout_mask` may also be a `(seed, offset)` pair of ints: the keep mask
+    is then drawn inside the library (Philox4x32-10, defined in
+    include/acct_fa.h) instead of being read from a [B,N,Sq,Sk] tensor, the
+    same way in forward and backward; `keep_prob` must be given.
   * dq, dk, dv come back in q's dtype directly (the reference returns fp32
     and casts to fp16 in bprop, flash_attention_impl.py:121-123).
 """
@@ -90,21 +94,29 @@ def _classify_mask(attn_mask, Sq, Sk):
     return kind, out
 
 
+def _is_seed_pair(x):
+    return isinstance(x, (tuple, list)) and len(x) == 2 and all(isinstance(t, int) for t in x)
+
+
 def _prepare_dropout(dropout_mask, keep_prob):
-    """Returns (uint8 mask or None, keep_prob)."""
+    """Returns (uint8 mask or None, keep_prob, (seed, offset) or None)."""
     if dropout_mask is None:
-        return None, 1.0
+        return None, 1.0, None
+    if _is_seed_pair(dropout_mask):
+        if keep_prob is None:
+            raise ValueError("a (seed, offset) dropout_mask needs keep_prob")
+        return None, float(keep_prob), (int(dropout_mask[0]), int(dropout_mask[1]))
     if dropout_mask.dtype in (torch.uint8, torch.bool):
         d8 = dropout_mask.contiguous()
         d8 = d8.view(torch.uint8) if d8.dtype == torch.bool else d8
         if keep_prob is None:
             raise ValueError("a uint8/bool dropout_mask needs keep_prob")
-        return d8, float(keep_prob)
+        return d8, float(keep_prob), None
     # the reference's form: fp16 {0, 1/keep_prob} (layer/flash_attention.py:198-203)
     if keep_prob is None:
         mx = float(dropout_mask.max())
         keep_prob = 1.0 / mx if mx > 0 else 1.0
-    return dropout_mask.ne(0).to(torch.uint8), float(keep_prob)
+    return dropout_mask.ne(0).to(torch.uint8), float(keep_prob), None
 
 
 def _build_params(q, k, v, attn_mask, dropout_mask, alibi_mask, prev_block_num, next_block_num, scale, keep_prob,
@@ -115,12 +127,13 @@ def _build_params(q, k, v, attn_mask, dropout_mask, alibi_mask, prev_block_num, 
         # a compact tile only ever touches diagonal blocks (attention.py:363-365,
         # flash_attention_fwd.py:353-356): blocks right of the diagonal stay visible
         kind, m8 = _capi.MASK_TILE_U8, torch.triu(torch.ones(128, 128, dtype=torch.uint8, device=q.device), diagonal=1)
-    d8, keep = _prepare_dropout(dropout_mask, keep_prob)
+    d8, keep, seed = _prepare_dropout(dropout_mask, keep_prob)
     if alibi_mask is not None and alibi_mask.dtype != q.dtype:
         alibi_mask = alibi_mask.to(q.dtype)
     return _capi.make_params(q, k, v, scale=scale, keep_prob=keep, prev_block_num=prev_block_num,
                              next_block_num=next_block_num, mask_kind=kind, attn_mask=m8, drop_mask=d8,
-                             alibi=alibi_mask, row_block_prefix=row_block_prefix)
+                             alibi=alibi_mask, row_block_prefix=row_block_prefix,
+                             drop_seed=None if seed is None else seed[0], drop_offset=0 if seed is None else seed[1])
 
 
 def _rows_contiguous(t):
@@ -161,7 +174,7 @@ def get_flash_attention_grad(prev_block_num=65536, next_block_num=65536, tiling_
         p = _build_params(q, k, v, attn_mask, dropout_mask, alibi_mask, prev_block_num, next_block_num, scale, keep_prob,
                           row_block_prefix)
         dq, dk, dv = _capi.fa_bwd(p, q, k, v, output, dout, rowsum)
-        zeros = tuple(None if t is None else torch.zeros_like(t) for t in (attn_mask, dropout_mask, alibi_mask))
+        zeros = tuple(torch.zeros_like(t) if torch.is_tensor(t) else None for t in (attn_mask, dropout_mask, alibi_mask))
         return (dq, dk, dv) + zeros
 
     return bprop

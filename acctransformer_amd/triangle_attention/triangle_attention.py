@@ -50,23 +50,26 @@ class TriangleAttention(torch.nn.Module):
         self._fused = block_size % 128 == 0
         self._op = get_flash_attention(scale=1.0, keep_prob=self.keep_prob,
                                        row_block_prefix=block_size if self._fused else 0)
+        self._calls = 0                               # one fresh dropout mask per training call
 
     def forward(self, query, key, value, attention_mask):
         bsz, head_num, seq_len, _ = query.shape
-        if self.enable_dropout and self.training:
-            drop_mask = (torch.rand((bsz, head_num, seq_len, seq_len), device=query.device) < self.keep_prob).to(torch.uint8)
-        else:
-            drop_mask = None
+        # dropout: no mask tensor, the library draws the keep decisions from a (seed, offset) pair
+        dropping = self.enable_dropout and self.training
+        seed = (torch.initial_seed() ^ 0x7F4A7C15F39CC060) & 0xFFFFFFFFFFFFFFFF
+        call = self._calls
+        if dropping:
+            self._calls += 1
         if self._fused:
-            o, _ = self._op(query, key, value, attention_mask, drop_mask, None)
+            o, _ = self._op(query, key, value, attention_mask, (seed, call & 0xFFFFFFFF) if dropping else None, None)
             return o
         # block_size off the 128 grid: one launch per row block on sliced views (`:137-163`)
         out = torch.empty_like(query)
-        for q_begin in range(0, seq_len, self.block_size):
+        for blk, q_begin in enumerate(range(0, seq_len, self.block_size)):
             q_end = min(q_begin + self.block_size, seq_len)
             kv_end = q_end
             cur_mask = attention_mask[:, q_begin:q_end, :kv_end].contiguous()
-            cur_drop = None if drop_mask is None else drop_mask[:, :, q_begin:q_end, :kv_end].contiguous()
+            cur_drop = (seed, (call * 4096 + blk) & 0xFFFFFFFF) if dropping else None    # every row block its own stream
             o, _ = self._op(query[:, :, q_begin:q_end], key[:, :, :kv_end], value[:, :, :kv_end], cur_mask, cur_drop, None)
             out[:, :, q_begin:q_end] = o
         return out

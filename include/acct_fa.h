@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define ACCT_FA_VERSION 100
+#define ACCT_FA_VERSION 101
 
 /* error codes (0 = success) */
 #define ACCT_OK          0
@@ -87,13 +87,27 @@ typedef struct acct_fa_params {
   const uint8_t* attn_mask;      /* per mask_kind; NULL when NONE / CAUSAL */
   const uint8_t* drop_mask;      /* uint8 [B,N,Sq,Sk] of {0,1}, contiguous; NULL = no dropout */
   const void*    alibi;          /* dtype, see strides; NULL = none (T/attention.py:347-355) */
+  /* Counter-based dropout (fields added in version 101): with drop_philox != 0, drop_mask == NULL and
+     keep_prob < 1 the keep mask is never materialised by the caller -- the library derives it from
+     (drop_seed, drop_offset) with Philox4x32-10, the same way in forward and backward.  It stands in
+     for the DropoutGenMask / DropoutDoMask chain of the reference layer (L/flash_attention.py:198-203),
+     which draws a [B,N,Sq,Sk] mask per call.  Definition (so that a caller or a test can rebuild the mask):
+       key     = (low 32 bits of drop_seed, high 32 bits of drop_seed)
+       counter = (i, 2*(j/32) + (j/4)%2, b*N + h, drop_offset)           i = query row, j = key column
+       byte    = byte 4*((j/8)%4) + j%4 of the 16 output bytes (word 0 first, little endian)
+       keep[b,h,i,j] = byte < T,  T = round(256 * keep_prob) clamped to 1..256
+     and kept probabilities are scaled by 256 / T (the reciprocal of the probability actually used).
+     Callers advance drop_offset (or change drop_seed) for every call that must draw a fresh mask. */
+  uint64_t drop_seed;
+  uint32_t drop_offset;
+  int32_t  drop_philox;
 } acct_fa_params;
 
 /* Forward: replaces the `flash_attention` TBE custom op, T/flash_attention_fwd.py:498-530
  * (outputs `output` and `rowsum`, T/flash_attention_impl.py:129-154).
  * O is [B,N,Sq,D] in p->dtype with p->o_stride; LSE is fp32 [B,N,Sq] contiguous
  * (L = m + ln l, T/flash_attention_fwd.py:302-306).  `workspace` must hold
- * acct_fa_fwd_workspace_bytes(p) bytes (0 unless mask_kind == DENSE_U8). */
+ * acct_fa_fwd_workspace_bytes(p) bytes (0 unless mask_kind == DENSE_U8 or dropout is on). */
 int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE,
                 void* workspace, size_t workspace_bytes, void* stream);
 size_t acct_fa_fwd_workspace_bytes(const acct_fa_params* p);

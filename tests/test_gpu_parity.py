@@ -23,6 +23,7 @@ from acctransformer_amd.flash_attention.ops.flash_attention.flash_attention_impl
     get_flash_attention, get_flash_attention_grad)
 from acctransformer_amd.triangle_attention.triangle_attention import TriangleAttention
 from golden_cases import load_cases
+from oracle import philox_dropout as phx
 from oracle import unfused_attention as orc
 
 pytestmark = pytest.mark.gpu
@@ -42,13 +43,13 @@ def _np(t):
 
 
 def _run(q, k, v, dO=None, *, scale, mask_kind=_capi.MASK_NONE, attn_mask=None, drop_mask=None, keep_prob=1.0,
-         alibi=None, prev=65536, nxt=65536, prefix=0):
+         alibi=None, prev=65536, nxt=65536, prefix=0, drop_seed=None, drop_offset=0):
     """One forward (and backward) through the C ABI on device copies of the inputs."""
     dev = lambda t: None if t is None else (torch.from_numpy(t) if isinstance(t, np.ndarray) else t).to(DEV)
     qd, kd, vd = dev(q), dev(k), dev(v)
     p = _capi.make_params(qd, kd, vd, scale=scale, keep_prob=keep_prob, prev_block_num=prev, next_block_num=nxt,
                           mask_kind=mask_kind, attn_mask=dev(attn_mask), drop_mask=dev(drop_mask), alibi=dev(alibi),
-                          row_block_prefix=prefix)
+                          row_block_prefix=prefix, drop_seed=drop_seed, drop_offset=drop_offset)
     o, lse = _capi.fa_fwd(p, qd)
     grads = None
     if dO is not None:
@@ -366,6 +367,45 @@ def test_layer_dropout_uses_one_mask_forward_and_backward():
     r = _np(o)[..., 0]
     assert abs(r.mean() - 1.0) < 0.05 and r.std() > 0.01
     assert np.allclose(_np(layer.eval()(q, k, v)), 1.0, atol=2e-3)
+
+
+# ---- counter-based dropout: the library draws the keep mask from (seed, offset) -----------------
+@pytest.mark.parametrize("Sq, Sk, D, causal, keep", [(256, 256, 128, True, 0.9), (200, 333, 64, False, 0.75),
+                                                     (384, 1100, 128, False, 0.5), (130, 96, 80, False, 0.9)])
+def test_counter_based_dropout_equals_explicit_mask(Sq, Sk, D, causal, keep):
+    # the mask rebuilt on the CPU from the definition in the C header, fed back as an explicit drop_mask with
+    # the keep probability the library actually uses, must give the same bits; and both must match the oracle
+    B, N = 2, 3
+    seed, off = (0x5EED << 36) + 77, 3
+    q, k, v, dO = (_gen(s, 700 + i) for i, s in enumerate([(B, N, Sq, D), (B, N, Sk, D), (B, N, Sk, D), (B, N, Sq, D)]))
+    drop = phx.dropout_keep_mask(B, N, Sq, Sk, seed, off, keep)
+    keep_eff = phx.keep_threshold(keep) / 256.0
+    kw = dict(scale=D ** -0.5)
+    okw = dict(scale=D ** -0.5, drop_mask=drop, keep_prob=keep_eff)
+    if causal:
+        kw.update(mask_kind=_capi.MASK_CAUSAL, nxt=0)
+        okw.update(attn_mask=np.triu(np.ones((1, Sq, Sk), dtype=np.uint8), 1))
+    a = _run(q, k, v, dO, keep_prob=keep, drop_seed=seed, drop_offset=off, **kw)
+    b = _run(q, k, v, dO, keep_prob=keep_eff, drop_mask=drop, **kw)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    for x, y in zip(a[2], b[2]):
+        assert torch.equal(x, y)
+    _check_all(q, k, v, dO, okw, a)
+    # another offset is another mask
+    c = _run(q, k, v, scale=D ** -0.5, keep_prob=keep, drop_seed=seed, drop_offset=off + 1,
+             **({"mask_kind": _capi.MASK_CAUSAL, "nxt": 0} if causal else {}))
+    assert not torch.equal(a[0], c[0])
+
+
+def test_counter_based_dropout_zero_pattern_exact():
+    # V = I makes O[i, j] the dropped probability of key j: the zeros must sit exactly where the mask has them
+    B, N, S, D = 1, 2, 128, 128
+    seed, off = 987654321987, 0
+    q, k = _gen((B, N, S, D), 710), _gen((B, N, S, D), 711)
+    v = torch.eye(S, D, dtype=torch.float16).expand(B, N, S, D).contiguous()
+    o, _, _ = _run(q, k, v, scale=D ** -0.5, keep_prob=0.6, drop_seed=seed, drop_offset=off)
+    drop = phx.dropout_keep_mask(B, N, S, S, seed, off, 0.6)
+    assert np.array_equal(_np(o) == 0, drop == 0)
 
 
 def test_bprop_closure_signature():

@@ -48,7 +48,7 @@ def test_struct_mirror_matches_header_field_order():
         for part in decl.split(","):
             names.append(re.sub(r"\[\d+\]", "", part.strip().split()[-1]).lstrip("*"))
     assert names == [f[0] for f in _capi.AcctFaParams._fields_]
-    assert ctypes.sizeof(_capi.AcctFaParams) == 224
+    assert ctypes.sizeof(_capi.AcctFaParams) == 240
 
 
 def _params(**over):
@@ -159,12 +159,39 @@ def test_mask_classification():
 
 def test_dropout_mask_forms():
     d = torch.tensor([[0.0, 1.25], [1.25, 0.0]], dtype=torch.float16)
-    m8, keep = impl._prepare_dropout(d, None)
-    assert m8.tolist() == [[0, 1], [1, 0]] and np.isclose(keep, 0.8)
-    m8, keep = impl._prepare_dropout(torch.tensor([[1, 0]], dtype=torch.uint8), 0.9)
-    assert keep == 0.9
+    m8, keep, seed = impl._prepare_dropout(d, None)
+    assert m8.tolist() == [[0, 1], [1, 0]] and np.isclose(keep, 0.8) and seed is None
+    m8, keep, seed = impl._prepare_dropout(torch.tensor([[1, 0]], dtype=torch.uint8), 0.9)
+    assert keep == 0.9 and seed is None
     with pytest.raises(ValueError):
         impl._prepare_dropout(torch.tensor([[1, 0]], dtype=torch.uint8), None)
+    # a (seed, offset) pair asks the library to draw the mask itself
+    m8, keep, seed = impl._prepare_dropout((1234, 5), 0.75)
+    assert m8 is None and keep == 0.75 and seed == (1234, 5)
+    with pytest.raises(ValueError):
+        impl._prepare_dropout((1234, 5), None)
+
+
+def test_counter_based_dropout_fields_and_workspace():
+    lib = _capi.load()
+    assert lib.acct_version() >= 101
+    q = torch.zeros(2, 2, 128, 128, dtype=torch.float16)
+    p = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, keep_prob=0.9, drop_seed=(7 << 40) + 3, drop_offset=11)
+    assert (p.drop_seed, p.drop_offset, p.drop_philox) == ((7 << 40) + 3, 11, 1)
+    # keep bits by query row: 2 * ceil(Sk / 64) words per row; by key column 16 bytes per (q block, key)
+    rows = 2 * 2 * 128 * 4 * 4
+    assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p)) == rows
+    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p)) == 2 * (2 * 2 * 128 * 4) + rows + 2 * 2 * 1 * 128 * 16
+    # keep_prob = 1 switches dropout off whatever the seed
+    p1 = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, keep_prob=1.0, drop_seed=5)
+    assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p1)) == 0
+    # keep_prob < 1 with neither a mask nor a seed is refused
+    p2 = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, keep_prob=0.9)
+    buf = (ctypes.c_char * 64)()
+    assert lib.acct_fa_fwd(ctypes.byref(p2), ctypes.addressof(buf), ctypes.addressof(buf), None, 0, None) == -1
+    with pytest.raises(ValueError):
+        _capi.make_params(q, q.clone(), q.clone(), scale=1.0, keep_prob=0.9, drop_seed=1,
+                          drop_mask=torch.ones(2, 2, 128, 128, dtype=torch.uint8))
 
 
 # ---- the oracle still reproduces the committed fixtures -------------------------

@@ -11,6 +11,7 @@ import pytest
 import scipy.special
 import torch
 
+from oracle import philox_dropout as phx
 from oracle import unfused_attention as orc
 
 
@@ -309,3 +310,42 @@ def test_data_compare_hand_counts():
     assert ok and np.isclose(ratio, 0.002 / (2e-3 + 2e-3)) and np.isclose(mx, 0.002)
     ok, _, _ = orc.tolerance_gate(gt, gt + np.array([0.0, 0.0, 0.0021, 0.0]))
     assert not ok
+
+
+# ---- counter-based dropout mask ---------------------------------------------------
+def test_philox4x32_10_known_answers():
+    # the known-answer vectors shipped with the Random123 library (kat_vectors, "philox4x32 10")
+    kat = [((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+           ((0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+           ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
+            (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1))]
+    for ctr, key, want in kat:
+        got = phx.philox4x32_10(np.array(ctr, dtype=np.uint32), key)
+        assert tuple(int(x) for x in got) == want
+    # vectorised over leading dimensions = one call per counter
+    ctrs = np.array([k[0] for k in kat[:1]] * 3, dtype=np.uint32).reshape(3, 1, 4)
+    assert np.array_equal(phx.philox4x32_10(ctrs, (0, 0))[2, 0], np.array(kat[0][2], dtype=np.uint32))
+
+
+def test_dropout_keep_mask_layout_and_rate():
+    B, N, Sq, Sk = 2, 3, 40, 100
+    seed, off = (0xABCD << 32) | 0x1234, 9
+    m = phx.dropout_keep_mask(B, N, Sq, Sk, seed, off, 0.75)
+    assert m.shape == (B, N, Sq, Sk) and m.dtype == np.uint8 and set(np.unique(m)) <= {0, 1}
+    # element by element from the definition in the C header, with scalar calls
+    thr = phx.keep_threshold(0.75)
+    assert thr == 192
+    rng = np.random.default_rng(0)
+    for _ in range(50):
+        b, h, i, j = (int(rng.integers(n)) for n in (B, N, Sq, Sk))
+        out = phx.philox4x32_10(np.array([i, 2 * (j // 32) + (j // 4) % 2, b * N + h, off], dtype=np.uint32),
+                                (seed & 0xFFFFFFFF, seed >> 32))
+        t = 4 * ((j // 8) % 4) + j % 4
+        byte = (int(out[t // 4]) >> (8 * (t % 4))) & 0xFF
+        assert m[b, h, i, j] == (1 if byte < thr else 0)
+    # a different offset or seed gives a different mask; the keep rate is threshold / 256
+    assert not np.array_equal(m, phx.dropout_keep_mask(B, N, Sq, Sk, seed, off + 1, 0.75))
+    assert not np.array_equal(m, phx.dropout_keep_mask(B, N, Sq, Sk, seed + 1, off, 0.75))
+    big = phx.dropout_keep_mask(1, 4, 256, 256, 42, 0, 0.9)
+    assert abs(big.mean() - phx.keep_threshold(0.9) / 256) < 0.004
+    assert phx.keep_threshold(1.0) == 256 and phx.keep_threshold(0.001) == 1
