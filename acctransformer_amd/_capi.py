@@ -83,6 +83,9 @@ def load():
     lib.acct_last_error.restype = ctypes.c_char_p
     lib.acct_build_is_complete.argtypes = []
     lib.acct_build_is_complete.restype = ctypes.c_int
+    I64P = ctypes.POINTER(ctypes.c_int64)
+    lib.acct_fa_infer_shape.argtypes = [I64P, ctypes.c_int, I64P, ctypes.c_int, I64P, ctypes.c_int, I64P]
+    lib.acct_fa_infer_shape.restype = ctypes.c_int
     lib.acct_version.argtypes = []
     lib.acct_version.restype = ctypes.c_int
     _lib = lib
@@ -220,3 +223,13 @@ def fa_bwd(p, q, k, v, o, do, lse):
         _check(lib.acct_fa_bwd(ctypes.byref(p), _ptr(o), _ptr(do), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv),
                                _ptr(ws), nws, _stream(q)))
     return dq, dk, dv
+
+
+def infer_shape(q_shape, k_shape, v_shape):
+    """acct_fa_infer_shape: the output shape of the inference operator for these input shapes,
+    or AcctError when the reference's shape function would reject them."""
+    lib = load()
+    arr = lambda s: (ctypes.c_int64 * max(len(s), 1))(*s)
+    y = (ctypes.c_int64 * 4)()
+    _check(lib.acct_fa_infer_shape(arr(q_shape), len(q_shape), arr(k_shape), len(k_shape), arr(v_shape), len(v_shape), y))
+    return tuple(y[i] for i in range(len(q_shape)))

@@ -58,13 +58,18 @@ uint32_t philox_threshold(float keep_prob) {
 }
 
 // Checks that need no device: used by the entry points and by the workspace queries.
-int validate(const acct_fa_params* p) {
+int validate(const acct_fa_params* p, bool backward) {
   if (!p) return fail(ACCT_E_NULLPTR, "params is NULL");
   if (p->dtype != ACCT_F16 && p->dtype != ACCT_BF16) return fail(ACCT_E_DTYPE, "dtype %d is neither ACCT_F16 nor ACCT_BF16", p->dtype);
   if (p->B <= 0 || p->N <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->D <= 0)
     return fail(ACCT_E_SHAPE, "extents must be positive: B=%d N=%d Sq=%d Sk=%d D=%d", p->B, p->N, p->Sq, p->Sk, p->D);
   if (p->D > 256) return fail(ACCT_E_HEADDIM, "head_dim too large, reduce head_dim and try again. (D=%d > 256)", p->D);
-  if (p->D != 64 && p->D != 80 && p->D != 128) return fail(ACCT_E_HEADDIM, "head_dim %d not built; supported: 64, 80, 128", p->D);
+  const bool d_train = p->D == 64 || p->D == 80 || p->D == 128;
+  const bool d_infer = p->D == 40 || p->D == 160;           // forward only, no bias / dropout: the inference operator's head dims
+  if (!d_train && !(d_infer && !backward))
+    return fail(ACCT_E_HEADDIM, "head_dim %d not built; supported: 64, 80, 128 (forward and backward), 40, 160 (forward only)", p->D);
+  if (d_infer && (p->alibi || p->drop_mask || (p->drop_philox && p->keep_prob < 1.f)))
+    return fail(ACCT_E_HEADDIM, "head_dim %d is built without the bias and dropout variants", p->D);
   if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return fail(ACCT_E_PARAM, "scale must be positive and finite, got %g", (double)p->scale);
   if (!(p->keep_prob > 0.f && p->keep_prob <= 1.f)) return fail(ACCT_E_PARAM, "keep_prob must be in (0, 1], got %g", (double)p->keep_prob);
   if (p->prev_block_num < 0 || p->next_block_num < 0) return fail(ACCT_E_PARAM, "prev_block_num / next_block_num must be >= 0");
@@ -184,7 +189,7 @@ size_t acct_fa_bwd_workspace_bytes(const acct_fa_params* p) {
 
 int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, size_t workspace_bytes, void* stream) {
   g_err[0] = 0;
-  int rc = validate(p);
+  int rc = validate(p, false);
   if (rc) return rc;
   if (!O || !LSE) return fail(ACCT_E_NULLPTR, "O and LSE must be non-NULL");
   if ((uintptr_t)O & 7) return fail(ACCT_E_SHAPE, "O must be 8-byte aligned");
@@ -222,7 +227,7 @@ int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, s
 static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, const float* LSE, void* dQ, void* dK, void* dV,
                     void* workspace, size_t workspace_bytes, void* stream, int stages) {
   g_err[0] = 0;
-  int rc = validate(p);
+  int rc = validate(p, true);
   if (rc) return rc;
   const bool want_dq = stages & acct::kStageDq, want_dkdv = stages & acct::kStageDkDv;
   if (!O || !dO || !LSE || (want_dq && !dQ) || (want_dkdv && (!dK || !dV)))
@@ -288,6 +293,39 @@ int acct_fa_bwd_dq(const acct_fa_params* p, const void* O, const void* dO, const
 int acct_fa_bwd_dkdv(const acct_fa_params* p, const void* O, const void* dO, const float* LSE, void* dK, void* dV,
                      void* workspace, size_t workspace_bytes, void* stream) {
   return bwd_impl(p, O, dO, LSE, nullptr, dK, dV, workspace, workspace_bytes, stream, acct::kStageDkDv);
+}
+
+// Shape function of the inference operator.  Limits and accept / reject behaviour follow
+// infer/flash_attention/tik/op_proto/flash_attention_tik.cpp:20-193 of the reference.
+int acct_fa_infer_shape(const int64_t* q_dims, int q_rank, const int64_t* k_dims, int k_rank,
+                        const int64_t* v_dims, int v_rank, int64_t* y_dims) {
+  g_err[0] = 0;
+  if (!q_dims || !k_dims || !v_dims) return fail(ACCT_E_NULLPTR, "q_dims, k_dims and v_dims must be non-NULL");
+  if (q_rank != 3 && q_rank != 4) return fail(ACCT_E_SHAPE, "q must have 3 or 4 dimensions, got %d", q_rank);
+  if (k_rank != q_rank || v_rank != q_rank) return fail(ACCT_E_SHAPE, "k and v must have q's number of dimensions");
+  auto in_range = [](int64_t x, int64_t lo, int64_t hi) { return x >= lo && x <= hi; };
+  auto same = [&](int i) { return k_dims[i] == q_dims[i] && v_dims[i] == q_dims[i]; };
+  const int s = q_rank - 2;                                          // position of the sequence length
+  if (q_rank == 3) {
+    if (!in_range(q_dims[0], 1, 64) || !same(0)) return fail(ACCT_E_SHAPE, "batch*heads must be 1..64 and equal for q, k, v");
+  } else {
+    if (!in_range(q_dims[0], 1, 64) || !same(0)) return fail(ACCT_E_SHAPE, "batch must be 1..64 and equal for q, k, v");
+    if (!in_range(q_dims[1], 1, 4096) || !same(1)) return fail(ACCT_E_SHAPE, "heads must be 1..4096 and equal for q, k, v");
+  }
+  if (!in_range(q_dims[s], 1, 8192) || !in_range(k_dims[s], 1, 8192) || v_dims[s] != k_dims[s])
+    return fail(ACCT_E_SHAPE, "sequence lengths must be 1..8192 and equal for k and v");
+  const int64_t d = q_dims[s + 1];
+  if (q_rank == 3) {
+    // the reference checks the last dimension of a 3-D input with its batch*heads rule (1..64 and equal),
+    // op_proto/flash_attention_tik.cpp:104-112; the kernel builder then wants one of its head dims
+    // (tbe/impl/flash_attention_fwd.py:38,104-106).  Both are applied here.
+    if (!in_range(d, 1, 64) || !same(2)) return fail(ACCT_E_HEADDIM, "head dim of a 3-D input must be 1..64 and equal for q, k, v");
+  }
+  if ((d != 40 && d != 64 && d != 80 && d != 160) || !same(s + 1))
+    return fail(ACCT_E_HEADDIM, "head dim must be one of 40, 64, 80, 160 and equal for q, k, v");
+  if (y_dims)
+    for (int i = 0; i < q_rank; i++) y_dims[i] = q_dims[i];
+  return ACCT_OK;
 }
 
 }  // extern "C"

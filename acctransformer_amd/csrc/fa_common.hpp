@@ -227,18 +227,19 @@ ACCT_DEV void tile_store(ACCT_LDS char* buf, const u32x4 (&reg)[TileCfg<D, NT>::
 ACCT_DEV int swz3(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
 
 template <int D> struct SwzCfg {
-  static constexpr int KS = D / 16;             // 16-wide k-steps across the head dim
+  static constexpr int KS = (D + 15) / 16;      // 16-wide k-steps across the head dim (the last one half empty when D % 16 == 8)
   static constexpr int DB = (D + 31) / 32;      // 32-wide blocks across the head dim
   static constexpr int CPR = D / 8;             // valid 16-byte chunks per row
-  static constexpr int CH = D <= 64 ? 8 : 16;   // chunk slots per LDS row
+  static constexpr int CH = D <= 64 ? 8 : (D <= 128 ? 16 : 32);   // chunk slots per LDS row
   static constexpr int PITCH = CH * 16;
   static constexpr int RPI = 64 / CH;           // rows covered by one wave-wide DMA instruction
-  static ACCT_DEV int swz(int row) { return CH == 16 ? (swz3(row) | (row & 8)) : ((row >> 1) & 7); }
+  // (rows of 512 bytes wrap around the banks twice: the four-bit swizzle of the 256-byte rows serves them too)
+  static ACCT_DEV int swz(int row) { return CH >= 16 ? (swz3(row) | (row & 8)) : ((row >> 1) & 7); }
   // Transposed reads come in pairs, rows r..r+3 and r+8..r+11 with r % 16 < 8: the second row group has
   // the top swizzle bit set, so its slot differs in that bit.  Which way depends only on the 32-column
   // block db the read belongs to (chunk 4 db + 0..3), i.e. the distance is a compile-time constant.
   static constexpr int tr_hi(int db) {
-    return 8 * PITCH + (CH == 16 ? (((db >> 1) & 1) ? -128 : 128) : ((db & 1) ? -64 : 64));
+    return 8 * PITCH + (CH >= 16 ? (((db >> 1) & 1) ? -128 : 128) : ((db & 1) ? -64 : 64));
   }
 };
 

@@ -72,8 +72,15 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   for (int gq = 0; gq < QG; gq++) {
     const int row = min(wq0 + 32 * gq + l32, a.Sq - 1);     // rows past Sq repeat the last row; never stored
 #pragma unroll
-    for (int t = 0; t < C::KS; t++)
-      qf[gq][t] = *reinterpret_cast<const V8*>(qp + (int64_t)row * a.q_ss + 16 * t + 8 * g);
+    for (int t = 0; t < C::KS; t++) {
+      // D % 16 == 8: the upper half of the last k-step lies past the row; zeros there make the products
+      // ignore whatever the K tile holds in that slot
+      const bool inside = (D % 16 == 0) || 16 * t + 8 * g < D;
+      V8 z;
+#pragma unroll
+      for (int e = 0; e < 8; e++) z[e] = 0;
+      qf[gq][t] = inside ? *reinterpret_cast<const V8*>(qp + (int64_t)row * a.q_ss + 16 * t + 8 * g) : z;
+    }
   }
 
   // ---- per-lane LDS offsets (tile-invariant) ----
@@ -399,15 +406,17 @@ static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
   return hipGetLastError();
 }
 
-template <typename T, int D, int QG, int NW>
+// SIDE = false: the head dims of the inference operator, built without the bias and dropout variants
+template <typename T, int D, int QG, int NW, bool SIDE = true>
 static hipError_t launch_fwd_q(const FaArgs& a, hipStream_t st) {
   const bool bias = a.alibi != nullptr, drop = a.droprow != nullptr || a.dropcol != nullptr;
 #ifndef ACCT_DEV_BUILD
-  if (bias) return drop ? launch_fwd_t<T, D, QG, NW, true, true>(a, st) : launch_fwd_t<T, D, QG, NW, true, false>(a, st);
-  if (drop) return launch_fwd_t<T, D, QG, NW, false, true>(a, st);
-#else
-  if (bias || drop) return hipErrorNotSupported;       // development build: plain variants only
+  if constexpr (SIDE) {
+    if (bias) return drop ? launch_fwd_t<T, D, QG, NW, true, true>(a, st) : launch_fwd_t<T, D, QG, NW, true, false>(a, st);
+    if (drop) return launch_fwd_t<T, D, QG, NW, false, true>(a, st);
+  }
 #endif
+  if (bias || drop) return hipErrorNotSupported;       // (development build: plain variants only)
   return launch_fwd_t<T, D, QG, NW, false, false>(a, st);
 }
 
@@ -416,6 +425,11 @@ template <typename T, int D>
 static hipError_t launch_fwd_d(const FaArgs& a, int variant, hipStream_t st) {
   if (variant == 3) return launch_fwd_q<T, D, 1, 8>(a, st);
   return variant == 2 ? launch_fwd_q<T, D, 2, 4>(a, st) : launch_fwd_q<T, D, 1, 4>(a, st);
+}
+// head dims 40 and 160: 32 rows per wave only
+template <typename T, int D>
+static hipError_t launch_fwd_plain(const FaArgs& a, int variant, hipStream_t st) {
+  return variant == 3 ? launch_fwd_q<T, D, 1, 8, false>(a, st) : launch_fwd_q<T, D, 1, 4, false>(a, st);
 }
 
 #ifdef ACCT_DEV_BUILD
@@ -433,10 +447,14 @@ hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st)
     if (D == 128) return launch_fwd_d<f16, 128>(a, qg, st);
     if (D == 64) return launch_fwd_d<f16, 64>(a, qg, st);
     if (D == 80) return launch_fwd_d<f16, 80>(a, qg, st);
+    if (D == 40) return launch_fwd_plain<f16, 40>(a, qg, st);
+    if (D == 160) return launch_fwd_plain<f16, 160>(a, qg, st);
   } else {
     if (D == 128) return launch_fwd_d<bf16, 128>(a, qg, st);
     if (D == 64) return launch_fwd_d<bf16, 64>(a, qg, st);
     if (D == 80) return launch_fwd_d<bf16, 80>(a, qg, st);
+    if (D == 40) return launch_fwd_plain<bf16, 40>(a, qg, st);
+    if (D == 160) return launch_fwd_plain<bf16, 160>(a, qg, st);
   }
   return hipErrorInvalidValue;
 #endif

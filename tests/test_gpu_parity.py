@@ -21,6 +21,7 @@ from acctransformer_amd import _capi
 from acctransformer_amd.flash_attention.nn.layer.flash_attention import FlashAttention
 from acctransformer_amd.flash_attention.ops.flash_attention.flash_attention_impl import (
     get_flash_attention, get_flash_attention_grad)
+from acctransformer_amd.infer.flash_attention.tik.flash_attention_tik import flash_attention_tik
 from acctransformer_amd.triangle_attention.triangle_attention import TriangleAttention
 from golden_cases import load_cases
 from oracle import philox_dropout as phx
@@ -406,6 +407,54 @@ def test_counter_based_dropout_zero_pattern_exact():
     o, _, _ = _run(q, k, v, scale=D ** -0.5, keep_prob=0.6, drop_seed=seed, drop_offset=off)
     drop = phx.dropout_keep_mask(B, N, S, S, seed, off, 0.6)
     assert np.array_equal(_np(o) == 0, drop == 0)
+
+
+# ---- inference operator: y = softmax(q k^T) v, head dims 40 / 64 / 80 / 160 ---------------------
+@pytest.mark.parametrize("shape_q, Sk", [((2, 4, 300, 40), 520), ((2, 2, 256, 160), 256), ((1, 3, 77, 160), 1000),
+                                         ((6, 200, 64), 130), ((2, 2, 128, 80), 384), ((3, 130, 40), 64)])
+def test_inference_operator_matches_torch_fp32_form(shape_q, Sk):
+    # the golden form of the reference's inference test (tests/infer/flash_attention/tik/data_gen.py:32-34);
+    # unit-variance inputs without scaling give very peaked rows, so q is drawn smaller to exercise the softmax
+    shape_k = shape_q[:-2] + (Sk, shape_q[-1])
+    q = (_gen(shape_q, 800) * 0.3).to(torch.float16)
+    k, v = _gen(shape_k, 801), _gen(shape_k, 802)
+    y = flash_attention_tik(q.to(DEV), k.to(DEV), v.to(DEV))
+    assert y.shape == q.shape and y.dtype == torch.float16
+    _gate(_np(orc.torch_unfused_fwd_fp32(q, k, v)), y, what="y")
+    out = torch.empty_like(y)
+    assert flash_attention_tik(q.to(DEV), k.to(DEV), v.to(DEV), out) is out and torch.equal(out, y)
+
+
+def test_inference_operator_rejects_what_the_reference_rejects():
+    z = lambda *s: torch.zeros(*s, dtype=torch.float16, device=DEV)
+    with pytest.raises(_capi.AcctError):
+        flash_attention_tik(z(2, 2, 128, 128), z(2, 2, 128, 128), z(2, 2, 128, 128))      # head dim 128 is not in its list
+    with pytest.raises(_capi.AcctError):
+        flash_attention_tik(z(4, 128, 80), z(4, 128, 80), z(4, 128, 80))                  # 3-D last dimension > 64
+    with pytest.raises(TypeError):
+        flash_attention_tik(*(z(2, 2, 128, 64).to(torch.bfloat16) for _ in range(3)))
+
+
+@pytest.mark.parametrize("D, dtype", [(40, torch.float16), (160, torch.float16), (160, torch.bfloat16), (40, torch.bfloat16)])
+def test_forward_only_head_dims_with_masks(D, dtype):
+    # the forward kernel of the two extra head dims through the C ABI: scale, causal mask with block skip,
+    # dense mask, ragged lengths -- against the fp64 operator spec
+    B, N, Sq, Sk = 2, 2, 333, 460
+    tol = dict(atol=ATOL_BF16, rtol=RTOL_BF16) if dtype == torch.bfloat16 else {}
+    q, k, v = (_gen(s, 810 + i, dtype) for i, s in enumerate([(B, N, Sq, D), (B, N, Sk, D), (B, N, Sk, D)]))
+    rng = np.random.default_rng(9)
+    mask = (rng.random((B, Sq, Sk)) < 0.3).astype(np.uint8)
+    mask[:, :, 0] = 0
+    _check_all(q, k, v, None, dict(scale=D ** -0.5, attn_mask=mask),
+               _run(q, k, v, scale=D ** -0.5, mask_kind=_capi.MASK_DENSE_U8, attn_mask=mask), **tol)
+    S = 384
+    q, k, v = (_gen((B, N, S, D), 820 + i, dtype) for i in range(3))
+    tri = np.triu(np.ones((1, S, S), dtype=np.uint8), 1)
+    _check_all(q, k, v, None, dict(scale=D ** -0.5, attn_mask=tri),
+               _run(q, k, v, scale=D ** -0.5, mask_kind=_capi.MASK_CAUSAL, nxt=0), **tol)
+    with pytest.raises(_capi.AcctError) as e:
+        _run(q, k, v, _gen((B, N, S, D), 830, dtype), scale=1.0)
+    assert e.value.code == -4
 
 
 def test_bprop_closure_signature():

@@ -28,7 +28,8 @@ def test_library_exports_every_declared_symbol():
     lib = _capi.load()
     decl = re.findall(r"^\s*(?:int|size_t|const char\*)\s+(acct_\w+)\s*\(", _header(), flags=re.M)
     assert set(decl) >= {"acct_fa_fwd", "acct_fa_bwd", "acct_fa_bwd_dq", "acct_fa_bwd_dkdv",
-                         "acct_fa_fwd_workspace_bytes", "acct_fa_bwd_workspace_bytes", "acct_last_error", "acct_version"}
+                         "acct_fa_fwd_workspace_bytes", "acct_fa_bwd_workspace_bytes", "acct_last_error", "acct_version",
+                         "acct_fa_infer_shape", "acct_build_is_complete"}
     for name in decl:
         assert hasattr(lib, name), name
     m = re.search(r"#define ACCT_FA_VERSION (\d+)", _header())
@@ -92,6 +93,50 @@ def test_null_outputs_and_workspace_sizes():
     assert lib.acct_fa_bwd(ctypes.byref(p2), *([addr] * 6), None, 0, None) == -7
     # D and -LSE*log2e rows, block classes (padded to 256), key-column bitmaps: 16 bytes per (q block, key)
     assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p2)) == 2 * (2 * 2 * 128 * 4) + 256 + 1 * 1 * 128 * 16
+
+
+def test_infer_shape_function():
+    # accept / reject cases of the inference operator's shape function
+    # (infer/flash_attention/tik/op_proto/flash_attention_tik.cpp:20-193 of the reference)
+    ok = _capi.infer_shape
+    assert ok((2, 8, 100, 160), (2, 8, 300, 160), (2, 8, 300, 160)) == (2, 8, 100, 160)
+    assert ok((64, 4096, 1, 40), (64, 4096, 8192, 40), (64, 4096, 8192, 40)) == (64, 4096, 1, 40)
+    assert ok((64, 77, 64), (64, 5, 64), (64, 5, 64)) == (64, 77, 64)
+    assert ok((8, 100, 40), (8, 100, 40), (8, 100, 40)) == (8, 100, 40)
+    bad = [
+        (((65, 8, 100, 64),) * 3, -2),                                   # batch > 64
+        (((2, 4097, 100, 64),) * 3, -2),                                 # heads > 4096
+        (((2, 8, 8193, 64),) * 3, -2),                                   # sequence > 8192
+        (((2, 8, 100, 64), (2, 8, 50, 64), (2, 8, 51, 64)), -2),         # k and v lengths differ
+        (((2, 8, 100, 64), (2, 9, 100, 64), (2, 8, 100, 64)), -2),       # heads differ
+        (((2, 8, 100, 128),) * 3, -4),                                   # head dim not in {40, 64, 80, 160}
+        (((2, 8, 100, 64), (2, 8, 100, 80), (2, 8, 100, 64)), -4),       # head dims differ
+        (((8, 100, 80),) * 3, -4),                                       # 3-D: last dimension held to 1..64
+        (((65, 100, 64),) * 3, -2),                                      # 3-D: batch*heads > 64
+        (((100, 64),) * 3, -2), (((1, 2, 8, 100, 64),) * 3, -2),         # rank
+        (((2, 8, 100, 64), (8, 100, 64), (8, 100, 64)), -2),             # ranks differ
+        (((2, 8, 0, 64),) * 3, -2),
+    ]
+    for shapes, code in bad:
+        with pytest.raises(_capi.AcctError) as e:
+            ok(*shapes)
+        assert e.value.code == code, shapes
+    lib = _capi.load()
+    assert lib.acct_fa_infer_shape(None, 4, None, 4, None, 4, None) == -1
+
+
+def test_inference_head_dims_are_forward_only():
+    lib = _capi.load()
+    buf = (ctypes.c_char * 64)()
+    a = ctypes.addressof(buf)
+    for D in (40, 160):
+        q = torch.zeros(1, 2, 128, D, dtype=torch.float16)
+        p = _capi.make_params(q, q.clone(), q.clone(), scale=1.0)
+        # the forward accepts the head dim (the call gets past validation to the NULL output check: nothing is launched)
+        assert lib.acct_fa_fwd(ctypes.byref(p), None, None, None, 0, None) == -1
+        assert lib.acct_fa_bwd(ctypes.byref(p), *([a] * 6), None, 0, None) == -4
+        p2 = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, keep_prob=0.9, drop_seed=1)
+        assert lib.acct_fa_fwd(ctypes.byref(p2), None, None, None, 0, None) == -4
 
 
 def test_no_cpu_fallback():
