@@ -278,7 +278,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
                     if ((mbits >> (8 * e)) & 0xffu) x[4 * r4 + e] += kMaskFill * kLog2e;
                 }
               }
-              {
+              if ((causal && (kv0 + 63 > wq0)) || (kv0 + 64 > a.Sk)) {
                 // keys after the query (causal) or past Sk: P is exactly 0
                 int vis = a.Sk - 1 - kv0 - 32 * c - 4 * g;
                 if (causal) vis = min(vis, qrow - kv0 - 32 * c - 4 * g);
@@ -492,7 +492,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   auto stage_bias = [&](int cn) { bias_tile_dma<T, false>(alibip, a.al_sq, cn * 32, a.Sq, wk0, a.Sk, bias_lds); };
 
   // per-chunk predicates of this pair (chunk = 32 query rows; two per staged tile)
-  auto classify = [&](int cidx, bool& act, bool& apply_mask, bool& edge) {
+  auto classify = [&](int cidx, bool& act, bool& apply_mask, bool& edge, bool& limits) {
     const int qc0 = cidx * 32, qt0 = (cidx >> 1) * 64, qb = cidx >> 2;
     act = (wkb - a.next_blk <= qb) && (qb <= wkb + a.prev_blk) && (wk0 < a.Sk);
     if (causal) act = act && (qt0 + 63 >= wk0);
@@ -505,7 +505,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     } else if (MASKT && a.mask_kind == kMaskTile) {
       apply_mask = wkb == qb;
     }
-    edge = BIAS || DROP || apply_mask || (causal && (wk0 + 63 > qc0)) || (wk0 + 64 > a.Sk) || (qc0 + 32 > a.Sq);
+    limits = (causal && (wk0 + 63 > qc0)) || (wk0 + 64 > a.Sk) || (qc0 + 32 > a.Sq);   // some (row, key) of the chunk is absent
+    edge = BIAS || DROP || apply_mask || limits;
   };
 
   if (i_lo <= i_hi) {
@@ -530,8 +531,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
       if ((n & 1) && (n >> 1) < i_hi) stage((n >> 1) + 1, smem + ((((n >> 1) + 1 - i_lo) & 1) * STAGEB));
       const int cidx = krole ? n - 1 : n;             // the chunk this wave works on in this step
       if (cidx >= c_lo && cidx <= c_hi) {
-        bool act, apply_mask, edge;
-        classify(cidx, act, apply_mask, edge);
+        bool act, apply_mask, edge, limits;
+        classify(cidx, act, apply_mask, edge, limits);
         if (act) {
           const int c = cidx & 1, qc0 = cidx * 32;
           // Per-lane LDS offsets are re-derived in every step (a handful of VALU ops) rather than
@@ -594,14 +595,17 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
               // (row, key) is set; -inf where the key comes after the query (causal) or where the key
               // or the query row does not exist (the probability is exactly 0 either way).
               if (BIAS && bias_staged) {
-                const ACCT_LDS char* bl = bias_lds + g * 512 + l32 * 2;     // row 4g, key l32 of the staged tile
+                // transposed reads of the row-major tile: each hands a lane the four consecutive rows
+                // 8i + 4g .. +3 of its key column (a 16-lane group covers 4 rows x 16 keys and supplies the
+                // addresses of that block's 8-byte pieces)
+                const ACCT_LDS char* bl = bias_lds + (4 * g + ((lane & 15) >> 2)) * 128 + ((lane >> 4) & 1) * 32 + (lane & 3) * 8;
 #pragma unroll
                 for (int gk = 0; gk < 2; gk++)
 #pragma unroll
-                  for (int r = 0; r < 16; r++) {
-                    const T bv = *reinterpret_cast<const ACCT_LDS T*>(bl + (8 * (r >> 2) + (r & 3)) * 128 + gk * 64);
-                    t0[gk][r] += (float)bv * a.inv_scale;
-                    if ((r & 7) == 7) asm volatile("" ::: "memory");
+                  for (int i = 0; i < 4; i++) {
+                    const typename E::V4 bv = __builtin_bit_cast(typename E::V4, lds_read_tr(bl + i * 8 * 128 + gk * 64));
+#pragma unroll
+                    for (int e = 0; e < 4; e++) t0[gk][4 * i + e] += (float)bv[e] * a.inv_scale;
                   }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // tile consumed: stage the next chunk's
                 if (n < c_hi) stage_bias(n + 1);
@@ -637,6 +641,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
                   }
                 }
               }
+              if (limits)
 #pragma unroll
               for (int gk = 0; gk < 2; gk++) {
                 const int kv = wk0 + 32 * gk + l32;

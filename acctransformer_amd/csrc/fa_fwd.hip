@@ -106,9 +106,10 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   }
 
   // Scores stay in raw q.k units (exp2 argument = s * scale*log2e - m * scale*log2e, one FMA) unless a
-  // bias is added, in which case they are converted to log2 units first.
-  const float cmul = BIAS ? 1.0f : a.scale_log2e;
-  const float madd = BIAS ? kMaskFill * kLog2e : a.mask_add_raw;   // the additive -10000 in the units of s
+  // bias is added, in which case they become scale*s + bias first (one mixed-precision FMA per score:
+  // the fp16 / bf16 bias is an operand as it is).
+  const float cmul = BIAS ? kLog2e : a.scale_log2e;
+  const float madd = BIAS ? kMaskFill : a.mask_add_raw;            // the additive -10000 in the units of s
   const float lazy_thr = 8.0f / cmul;                              // 8 octaves, in the units of s
   const int mb = a.mask_sb ? b : 0;
   const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
@@ -220,7 +221,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
                 for (int r4 = 0; r4 < 4; r4++)
 #pragma unroll
                   for (int e = 0; e < 4; e++)
-                    s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale_log2e, (float)bv[c][r4][e] * kLog2e);
+                    s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale, (float)bv[c][r4][e]);
             } else {
 #pragma unroll
               for (int c = 0; c < 2; c++)
@@ -231,7 +232,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
                   load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
 #pragma unroll
                   for (int e = 0; e < 4; e++)
-                    s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale_log2e, bias[e] * kLog2e);
+                    s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale, bias[e]);
                 }
             }
           }
@@ -356,7 +357,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   // LDS region (pitch 2D+16 keeps the 8-byte writes of 16 rows on distinct banks) so that the
   // global stores are whole rows. ----
   T* op = (T*)a.o + b * a.o_sb + h * a.o_sh;
-  const float mnat = BIAS ? kLn2 : a.scale;
+  const float mnat = BIAS ? 1.0f : a.scale;
   constexpr int OPITCH = C::DB * 64 + 16;
   ACCT_LDS char* obuf = smem + wave * (32 * OPITCH);
 #pragma unroll
