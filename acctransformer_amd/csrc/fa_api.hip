@@ -143,6 +143,11 @@ size_t flag_bytes(const acct_fa_params* p) {
   const size_t MB = p->mask_stride_b ? p->B : 1;
   return align_up(MB * (size_t)((p->Sq + 127) / 128) * (size_t)((p->Sk + 127) / 128), 256);
 }
+// classify the blocks of a dense mask; fills a.blkflags
+hipError_t prepare_mask(acct::FaArgs& a, const acct_fa_params* p, uint8_t* flags, hipStream_t st) {
+  a.blkflags = flags;
+  return acct::launch_mask_blocks(a, flags, p->mask_stride_b ? p->B : 1, st);
+}
 
 // per-key-column bitmaps of the mixed blocks of a dense mask (backward only): 16 bytes per (q block, key)
 size_t colbit_bytes(const acct_fa_params* p) {
@@ -204,8 +209,7 @@ int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, s
   acct::FaArgs a = make_args(p);
   a.o = O; a.lse = LSE;
   if (p->mask_kind == ACCT_MASK_DENSE_U8) {
-    a.blkflags = (const uint8_t*)workspace;
-    hipError_t e = acct::launch_mask_blocks(a, (uint8_t*)workspace, p->mask_stride_b ? p->B : 1, st);
+    hipError_t e = prepare_mask(a, p, (uint8_t*)workspace, st);
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
   }
   if (dropout_on(p)) {
@@ -251,11 +255,9 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
   a.nlse = (float*)((char*)workspace + stat_bytes);
   if (p->mask_kind == ACCT_MASK_DENSE_U8) {
     uint8_t* flags = (uint8_t*)workspace + 2 * stat_bytes;
-    a.blkflags = flags;
-    if (want_dq || stages == acct::kStageDkDv) {   // the dkdv-only call re-derives the flags: the mask may have been edited since
-      hipError_t e = acct::launch_mask_blocks(a, flags, p->mask_stride_b ? p->B : 1, st);
-      if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
-    }
+    // (the dkdv-only call re-derives the flags as well: the mask may have been edited since)
+    hipError_t e = prepare_mask(a, p, flags, st);
+    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
   }
   if (want_dkdv && (p->mask_kind == ACCT_MASK_DENSE_U8 || p->mask_kind == ACCT_MASK_TILE_U8)) {
     uint8_t* flags = (uint8_t*)workspace + 2 * stat_bytes;          // (no flags for the tile kind: flag_bytes = 0)

@@ -85,8 +85,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
         if (fl[(int64_t)qb * a.Tc + (j >> 1)] != kBlkSkip) return false;
       return true;
     };
-    while (j_lo <= j_hi && dead(j_lo)) j_lo++;
-    while (j_lo <= j_hi && dead(j_hi)) j_hi--;
+    trim_dead_tiles(j_lo, j_hi, lane, dead);
   }
   const int wqb = wq0 / 128;
   const int wkv_limit = a.row_prefix ? (wq0 / a.row_prefix + 1) * a.row_prefix : 0x7fffffff;
@@ -163,7 +162,12 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
+    // block classes of a dense mask are fetched one tile ahead: the load has a whole tile to come back
+    const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
+    uint32_t fl_next = flrow ? flrow[j_lo >> 1] : 0u;
     for (int j = j_lo; j <= j_hi; j++) {
+      const uint32_t fl_cur = fl_next;
+      if (flrow && j < j_hi) fl_next = flrow[(j + 1) >> 1];
       const int buf = (j - j_lo) & 1;
       ACCT_LDS char* kbuf = smem + buf * 2 * TILEB;
       ACCT_LDS char* vbuf = kbuf + TILEB;
@@ -184,9 +188,8 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
       act = act && (kv0 < wkv_limit);
       bool apply_mask = false;
       if (MASKT && a.mask_kind == kMaskDense && act) {
-        const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + wqb) * a.Tc + kvb];
-        act = f != kBlkSkip;
-        apply_mask = f == kBlkApply;
+        act = fl_cur != kBlkSkip;
+        apply_mask = fl_cur == kBlkApply;
       } else if (MASKT && a.mask_kind == kMaskTile) {
         apply_mask = wqb == kvb;
       }
@@ -421,8 +424,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
         if (fl[(int64_t)(i >> 1) * a.Tc + kb] != kBlkSkip) return false;
       return true;
     };
-    while (i_lo <= i_hi && dead(i_lo)) i_lo++;
-    while (i_lo <= i_hi && dead(i_hi)) i_hi--;
+    trim_dead_tiles(i_lo, i_hi, lane, dead);
   }
   const int wkb = wk0 / 128;
 
@@ -492,16 +494,15 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   auto stage_bias = [&](int cn) { bias_tile_dma<T, false>(alibip, a.al_sq, cn * 32, a.Sq, wk0, a.Sk, bias_lds); };
 
   // per-chunk predicates of this pair (chunk = 32 query rows; two per staged tile)
-  auto classify = [&](int cidx, bool& act, bool& apply_mask, bool& edge, bool& limits) {
+  auto classify = [&](int cidx, uint32_t fl, bool& act, bool& apply_mask, bool& edge, bool& limits) {
     const int qc0 = cidx * 32, qt0 = (cidx >> 1) * 64, qb = cidx >> 2;
     act = (wkb - a.next_blk <= qb) && (qb <= wkb + a.prev_blk) && (wk0 < a.Sk);
     if (causal) act = act && (qt0 + 63 >= wk0);
     if (a.row_prefix) act = act && (wk0 < (qt0 / a.row_prefix + 1) * a.row_prefix);
     apply_mask = false;
     if (MASKT && a.mask_kind == kMaskDense && act) {
-      const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + qb) * a.Tc + wkb];
-      act = f != kBlkSkip;
-      apply_mask = f == kBlkApply;
+      act = fl != kBlkSkip;                            // class of block (qb, wkb), fetched one step ahead
+      apply_mask = fl == kBlkApply;
     } else if (MASKT && a.mask_kind == kMaskTile) {
       apply_mask = wkb == qb;
     }
@@ -521,6 +522,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     // publishes it and accumulates dV; the K role picks up P of chunk n-1.  One barrier per step,
     // nothing is carried across it in registers.
     const int c_lo = 2 * i_lo, c_hi = 2 * i_hi + 1;
+    const uint8_t* flcol = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + (int64_t)mb * a.Tr * a.Tc + wkb : nullptr;
+    uint32_t fl_next = flcol ? flcol[(int64_t)(c_lo >> 2) * a.Tc] : 0u;
 #ifdef ACCT_TRACE
 #define TR(k) if (blockIdx.x == ACCT_TRACE && lane == 0 && n - c_lo < 96) ((unsigned long long*)((char*)a.delta + 2 * (size_t)a.B * a.N * a.Sq * 4))[((wave * 96) + (n - c_lo)) * 8 + (k)] = __builtin_amdgcn_s_memtime()
 #else
@@ -532,7 +535,9 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
       const int cidx = krole ? n - 1 : n;             // the chunk this wave works on in this step
       if (cidx >= c_lo && cidx <= c_hi) {
         bool act, apply_mask, edge, limits;
-        classify(cidx, act, apply_mask, edge, limits);
+        const uint32_t fl_cur = fl_next;
+        if (flcol && cidx < c_hi) fl_next = flcol[(int64_t)((cidx + 1) >> 2) * a.Tc];
+        classify(cidx, fl_cur, act, apply_mask, edge, limits);
         if (act) {
           const int c = cidx & 1, qc0 = cidx * 32;
           // Per-lane LDS offsets are re-derived in every step (a handful of VALU ops) rather than

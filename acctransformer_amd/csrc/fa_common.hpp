@@ -152,6 +152,25 @@ ACCT_DEV void wg_map(int id, int BH, int n_tiles, int& bh, int& rank) {
   }
 }
 
+// Shrinks the tile range [lo, hi] from both ends while dead(tile) holds.  The 64 lanes of the wave test 64
+// tiles at a time (one round trip to memory per 64 tiles instead of one per tile); every wave of the
+// workgroup arrives at the same range.
+template <typename F>
+ACCT_DEV void trim_dead_tiles(int& lo, int& hi, int lane, F dead) {
+  while (lo <= hi) {
+    const int j = lo + lane;
+    const uint64_t live = __ballot(j > hi || !dead(j));
+    if (live) { lo += __builtin_ctzll(live); break; }
+    lo += 64;
+  }
+  while (lo <= hi) {
+    const int j = hi - lane;
+    const uint64_t live = __ballot(j < lo || !dead(j));
+    if (live) { hi -= __builtin_ctzll(live); break; }
+    hi -= 64;
+  }
+}
+
 // four consecutive mask / dropout bytes starting at column kv of a row
 ACCT_DEV uint32_t load_u8x4(const uint8_t* row, int kv, int limit, bool vec_ok) {
   if (vec_ok && kv + 4 <= limit) return *reinterpret_cast<const uint32_t*>(row + kv);

@@ -60,8 +60,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
         if (fl[(int64_t)qb * a.Tc + (j >> 1)] != kBlkSkip) return false;
       return true;
     };
-    while (j_lo <= j_hi && dead(j_lo)) j_lo++;
-    while (j_lo <= j_hi && dead(j_hi)) j_hi--;
+    trim_dead_tiles(j_lo, j_hi, lane, dead);
   }
   const int wqb = wq0 / 128;                                // 128-block of this wave's rows
   const int wkv_limit = a.row_prefix ? (wq0 / a.row_prefix + 1) * a.row_prefix : 0x7fffffff;   // keys past it are absent
@@ -143,8 +142,13 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
 #else
 #define TR(k)
 #endif
+    // block classes of a dense mask are fetched one tile ahead: the load has a whole tile to come back
+    const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
+    uint32_t fl_next = flrow ? flrow[j_lo >> 1] : 0u;
     for (int j = j_lo; j <= j_hi; j++) {
       TR(0);
+      const uint32_t fl_cur = fl_next;
+      if (flrow && j < j_hi) fl_next = flrow[(j + 1) >> 1];
       const int buf = (j - j_lo) & 1;
       ACCT_LDS char* kbuf = smem + buf * 2 * TILEB;
       ACCT_LDS char* vbuf = kbuf + TILEB;
@@ -165,9 +169,8 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
       act = act && (kv0 < wkv_limit);
       bool apply_mask = false;
       if (MASKT && a.mask_kind == kMaskDense && act) {
-        const uint8_t f = a.blkflags[((int64_t)mb * a.Tr + wqb) * a.Tc + kvb];
-        act = f != kBlkSkip;
-        apply_mask = f == kBlkApply;
+        act = fl_cur != kBlkSkip;
+        apply_mask = fl_cur == kBlkApply;
       } else if (MASKT && a.mask_kind == kMaskTile) {
         apply_mask = wqb == kvb;
       }
