@@ -522,6 +522,16 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     // publishes it and accumulates dV; the K role picks up P of chunk n-1.  One barrier per step,
     // nothing is carried across it in registers.
     const int c_lo = 2 * i_lo, c_hi = 2 * i_hi + 1;
+    // offsets of the transposed fragments of d block db: kept across the steps where the registers allow
+    // (a fifth of the step's vector instructions otherwise), re-derived in every step in the bias variants
+    constexpr bool KEEP_TOFF = !BIAS;
+    int toff2_kept[2] = {0, 0};
+    if (KEEP_TOFF) {
+      const int trow = 4 * g + ((lane & 15) >> 2);
+      const int tchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+#pragma unroll
+      for (int db = 0; db < 2; db++) toff2_kept[db] = trow * C::PITCH + swz_off(4 * db + tchunk, C::swz(trow)) + 8 * (lane & 1);
+    }
     const uint8_t* flcol = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + (int64_t)mb * a.Tr * a.Tc + wkb : nullptr;
     uint32_t fl_next = flcol ? flcol[(int64_t)(c_lo >> 2) * a.Tc] : 0u;
 #ifdef ACCT_TRACE
@@ -549,11 +559,16 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
           int foff4[4];                               // row-major fragment of k-step t: row l32, chunk 2t + g
 #pragma unroll
           for (int t = 0; t < 4; t++) foff4[t] = (ln & 31) * C::PITCH + swz_off(2 * t + (ln >> 5), C::swz(ln & 31));
-          const int trow = 4 * (ln >> 5) + ((ln & 15) >> 2);
-          const int tchunk = 2 * ((ln >> 4) & 1) + ((ln & 3) >> 1);
-          int toff2[2];                               // transposed fragment of d block db
+          int toff2[2];
+          if (KEEP_TOFF) {
+            toff2[0] = toff2_kept[0];
+            toff2[1] = toff2_kept[1];
+          } else {
+            const int trow = 4 * (ln >> 5) + ((ln & 15) >> 2);
+            const int tchunk = 2 * ((ln >> 4) & 1) + ((ln & 3) >> 1);
 #pragma unroll
-          for (int db = 0; db < 2; db++) toff2[db] = trow * C::PITCH + swz_off(4 * db + tchunk, C::swz(trow)) + 8 * (ln & 1);
+            for (int db = 0; db < 2; db++) toff2[db] = trow * C::PITCH + swz_off(4 * db + tchunk, C::swz(trow)) + 8 * (ln & 1);
+          }
           ACCT_LDS char* qbuf = smem + (((cidx >> 1) - i_lo) & 1) * STAGEB;
           ACCT_LDS char* dobuf = qbuf + TILEB;
           const ACCT_LDS float* lbuf = (const ACCT_LDS float*)(qbuf + 2 * TILEB);
@@ -696,7 +711,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
                   for (int e = 0; e < 4; e++) {
                     float dpv = t0[gk][8 * hh + 4 * r4 + e];
                     if (DROP) dpv = ((dcw[gk] >> (16 * hh + 8 * r4 + e)) & 1u) ? dpv * a.inv_keep : 0.f;
-                    ds[4 * r4 + e] = (float)ph[4 * r4 + e] * (dpv - dv4[e]);
+                    // (an FMA with a zero addend keeps the fp16 -> fp32 conversion inside one mixed-precision instruction)
+                    ds[4 * r4 + e] = __builtin_fmaf((float)ph[4 * r4 + e], dpv - dv4[e], 0.0f);
                   }
                 }
                 bfr[gk][hh] = pack8<T>(ds);
