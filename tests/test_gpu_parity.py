@@ -457,6 +457,68 @@ def test_forward_only_head_dims_with_masks(D, dtype):
     assert e.value.code == -4
 
 
+def test_layer_dropout_follows_torch_seed_and_call_count():
+    # the layers hand the op (seed, offset): torch's seed makes a run repeatable, every training call
+    # draws a fresh mask, and the gradients see the mask of their own forward
+    B, N, S, D = 1, 2, 256, 64
+    q, k, v = (_gen((B, N, S, D), s).to(DEV) for s in (840, 841, 842))
+    torch.manual_seed(123)
+    a = FlashAttention(head_dim=D, dropout_rate=0.3).train()
+    a1, a2 = a(q, k, v), a(q, k, v)
+    assert not torch.equal(a1, a2)                      # second call, next offset
+    torch.manual_seed(123)
+    b = FlashAttention(head_dim=D, dropout_rate=0.3).train()
+    b._layer_id = a._layer_id                           # same layer identity = same stream
+    assert torch.equal(b(q, k, v), a1) and torch.equal(b(q, k, v), a2)
+    torch.manual_seed(124)
+    assert not torch.equal(FlashAttention(head_dim=D, dropout_rate=0.3).train()(q, k, v), a1)
+    # forward and backward of one call agree on the mask: with V = I the output is the dropped probability
+    # matrix, and dV = P_dropped^T dO must vanish exactly where a whole key column was dropped for every row
+    eye = torch.eye(S, D, dtype=torch.float16, device=DEV).expand(B, N, S, D).contiguous().requires_grad_(True)
+    layer = FlashAttention(head_dim=D, dropout_rate=0.5).train()
+    o = layer(q, k, eye)
+    o.backward(torch.ones_like(o))
+    kept_any = (o[..., :D] != 0).any(dim=2)             # key j < D kept by some row  <=>  column j of O non-zero
+    dv_rows = eye.grad[:, :, :D, :].abs().sum(dim=3) != 0
+    assert torch.equal(kept_any, dv_rows)
+
+
+@pytest.mark.parametrize("bs", [128, 200])
+def test_triangle_attention_training_dropout(bs):
+    # fused (block size on the 128 grid) and sliced path: same statistics, fresh mask per call
+    B, N, S, D = 1, 2, 512, 64
+    q, k = ((_gen((B, N, S, D), s) * 0.3).half().to(DEV) for s in (850, 851))
+    v = torch.ones(B, N, S, D, dtype=torch.float16, device=DEV)
+    mask = torch.triu(torch.ones(B, S, S, dtype=torch.float16, device=DEV), 1)
+    layer = TriangleAttention(block_size=bs, dropout_rate=0.25).train()
+    torch.manual_seed(7)
+    o1, o2 = layer(q, k, v, mask), layer(q, k, v, mask)
+    r = _np(o1)[..., 0]
+    # V = 1: every output is kept mass / keep probability; rows with many visible keys concentrate around 1
+    assert abs(r[:, :, 128:].mean() - 1.0) < 0.03 and r[:, :, 128:].std() > 0.005
+    assert not torch.equal(o1, o2)
+    assert np.allclose(_np(layer.eval()(q, k, v, mask)), 1.0, atol=2e-3)
+
+
+def test_counter_based_dropout_bf16_backward():
+    B, N, Sq, Sk, D = 1, 2, 192, 320, 128
+    seed, off, keep = 31337, 5, 0.8
+    q, k, v, dO = (_gen(s, 860 + i, torch.bfloat16) for i, s in enumerate([(B, N, Sq, D), (B, N, Sk, D), (B, N, Sk, D), (B, N, Sq, D)]))
+    drop = phx.dropout_keep_mask(B, N, Sq, Sk, seed, off, keep)
+    okw = dict(scale=D ** -0.5, drop_mask=drop, keep_prob=phx.keep_threshold(keep) / 256.0)
+    _check_all(q, k, v, dO, okw, _run(q, k, v, dO, scale=D ** -0.5, keep_prob=keep, drop_seed=seed, drop_offset=off),
+               atol=ATOL_BF16, rtol=RTOL_BF16)
+
+
+def test_inference_operator_at_its_length_limit():
+    # 8192 keys and queries, the operator's maximum (op_proto/flash_attention_tik.cpp:23), one head
+    S, D = 8192, 64
+    q = (_gen((1, S, D), 870) * 0.3).to(torch.float16)
+    k, v = _gen((1, S, D), 871), _gen((1, S, D), 872)
+    y = flash_attention_tik(q.to(DEV), k.to(DEV), v.to(DEV))
+    _gate(_np(orc.torch_unfused_fwd_fp32(q, k, v)), y, what="y at S = 8192")
+
+
 def test_bprop_closure_signature():
     B, N, S, D = 1, 2, 256, 128
     q, k, v, dO = (_gen((B, N, S, D), s).to(DEV) for s in (63, 64, 65, 66))
