@@ -4,9 +4,9 @@
 // (train/acctransformer/flash_attention/ops/flash_attention/flash_attention_fwd.py:308-474:
 // Q-outer / KV-inner loops, online softmax, O rescale, O/l and L = m + ln l).
 //
-// Work split: one workgroup (4 waves) owns 128*QG query rows of one (batch,
-// head); each wave owns 32*QG of them.  K and V tiles of 64 rows are staged
-// through LDS (double buffered) and shared by the 4 waves.  The wave computes
+// Work split: one workgroup (4 or 8 waves) owns 32*QG query rows per wave of one
+// (batch, head).  K and V tiles of 64 rows (128 in the variants without side
+// inputs) are staged through LDS (double buffered) and shared by the waves.  The wave computes
 // the TRANSPOSED score tile S^T = K Q^T with 32x32x16 MFMAs, so every lane
 // holds scores of a single query row (column l%32 of the MFMA C tile): the
 // online-softmax state (running max, running sum) is per lane, row
@@ -18,13 +18,16 @@
 
 namespace acct {
 
-template <typename T, int D, int QG, int NW, bool BIAS, bool DROP, bool MASKT>
+template <typename T, int D, int QG, int NW, bool BIAS, bool DROP, bool MASKT, int KT = 2>
 __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
+  static_assert(KT == 2 || (KT == 4 && !BIAS), "key tiles are 64 rows, or 128 rows in the variants without bias");
+  constexpr int BN = 32 * KT;                       // key rows per tile
+  constexpr int TPB = 128 / BN;                     // tiles per 128-column block
   using E = Elem<T>;
   using V8 = typename E::V8;
   using C = SwzCfg<D>;
   constexpr int BM = 32 * QG * NW;
-  constexpr int TILEB = 64 * C::PITCH;
+  constexpr int TILEB = BN * C::PITCH;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 buffers][K tile | V tile]; reused by the epilogue
 
@@ -47,17 +50,17 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   // ---- visible kv tiles of this block (128-block band; causal and row-prefix clip the top) ----
   const int qb_lo = q0 / 128, qb_hi = (q_end - 1) / 128;
   const int kvb_lo = max(0, qb_lo - a.prev_blk), kvb_hi = min(a.Tc - 1, qb_hi + a.next_blk);
-  int j_lo = kvb_lo * 2, j_hi = min(kvb_hi * 2 + 1, (a.Sk - 1) / 64);
+  int j_lo = kvb_lo * TPB, j_hi = min(kvb_hi * TPB + TPB - 1, (a.Sk - 1) / BN);
   const bool causal = a.mask_kind == kMaskCausal;
-  if (causal) j_hi = min(j_hi, (q_end - 1) / 64);
-  if (a.row_prefix) j_hi = min(j_hi, (((q_end - 1) / a.row_prefix + 1) * a.row_prefix - 1) / 64);
+  if (causal) j_hi = min(j_hi, (q_end - 1) / BN);
+  if (a.row_prefix) j_hi = min(j_hi, (((q_end - 1) / a.row_prefix + 1) * a.row_prefix - 1) / BN);
   if (MASKT && a.mask_kind == kMaskDense) {
     // tiles at either end whose 128x128 blocks are wholly masked for every row block of this workgroup are
     // not streamed at all (key padding: the padded tail of every sequence)
     const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc;
     auto dead = [&](int j) {
       for (int qb = qb_lo; qb <= qb_hi; qb++)
-        if (fl[(int64_t)qb * a.Tc + (j >> 1)] != kBlkSkip) return false;
+        if (fl[(int64_t)qb * a.Tc + j / TPB] != kBlkSkip) return false;
       return true;
     };
     trim_dead_tiles(j_lo, j_hi, lane, dead);
@@ -117,7 +120,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
                                                   : ((uintptr_t)a.mask & 3) == 0;
   const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
-  TileDma<T, D, 64, NW> kdma, vdma;
+  TileDma<T, D, BN, NW> kdma, vdma;
   kdma.plan(a.k_ss);
   vdma.plan(a.v_ss);
   // bias tiles of this wave's rows are staged through a wave-private LDS region one tile ahead
@@ -129,8 +132,8 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
       bias_tile_dma<T>(alibip, a.al_sq, wq0 + 32 * gq, a.Sq, jn * 64, a.Sk, bias_lds + gq * 4096);
   };
   if (j_lo <= j_hi) {
-    tile_dma<T, D, 64, NW>(kp, a.k_ss, j_lo * 64, a.Sk, smem);
-    tile_dma<T, D, 64, NW>(vp, a.v_ss, j_lo * 64, a.Sk, smem + TILEB);
+    tile_dma<T, D, BN, NW>(kp, a.k_ss, j_lo * BN, a.Sk, smem);
+    tile_dma<T, D, BN, NW>(vp, a.v_ss, j_lo * BN, a.Sk, smem + TILEB);
     if (BIAS && bias_staged && wq0 < a.Sq) stage_bias(j_lo);
     // A full wait the compiler can see: every load issued so far (Q fragments included) is complete, so
     // it places no vmcnt wait inside the loop -- such a wait would also stall on the next tile's DMA.
@@ -144,26 +147,26 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
 #endif
     // block classes of a dense mask are fetched one tile ahead: the load has a whole tile to come back
     const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
-    uint32_t fl_next = flrow ? flrow[j_lo >> 1] : 0u;
+    uint32_t fl_next = flrow ? flrow[j_lo / TPB] : 0u;
     for (int j = j_lo; j <= j_hi; j++) {
       TR(0);
       const uint32_t fl_cur = fl_next;
-      if (flrow && j < j_hi) fl_next = flrow[(j + 1) >> 1];
+      if (flrow && j < j_hi) fl_next = flrow[(j + 1) / TPB];
       const int buf = (j - j_lo) & 1;
       ACCT_LDS char* kbuf = smem + buf * 2 * TILEB;
       ACCT_LDS char* vbuf = kbuf + TILEB;
       if (j < j_hi) {                                       // next tile streams into the other buffer meanwhile
         ACCT_LDS char* nb = smem + (buf ^ 1) * 2 * TILEB;
-        if ((j + 2) * 64 <= a.Sk) {
-          kdma.issue(kp, a.k_ss, (j + 1) * 64, nb);
-          vdma.issue(vp, a.v_ss, (j + 1) * 64, nb + TILEB);
+        if ((j + 2) * BN <= a.Sk) {
+          kdma.issue(kp, a.k_ss, (j + 1) * BN, nb);
+          vdma.issue(vp, a.v_ss, (j + 1) * BN, nb + TILEB);
         } else {                                            // ragged last tile: clamped rows
-          tile_dma<T, D, 64, NW>(kp, a.k_ss, (j + 1) * 64, a.Sk, nb);
-          tile_dma<T, D, 64, NW>(vp, a.v_ss, (j + 1) * 64, a.Sk, nb + TILEB);
+          tile_dma<T, D, BN, NW>(kp, a.k_ss, (j + 1) * BN, a.Sk, nb);
+          tile_dma<T, D, BN, NW>(vp, a.v_ss, (j + 1) * BN, a.Sk, nb + TILEB);
         }
       }
-      const int kv0 = j * 64;
-      const int kvb = j >> 1;
+      const int kv0 = j * BN;
+      const int kvb = j / TPB;
       bool act = (kvb - a.next_blk <= wqb) && (wqb <= kvb + a.prev_blk) && (wq0 < a.Sq);
       if (causal) act = act && (kv0 <= wq_end - 1);
       act = act && (kv0 < wkv_limit);
@@ -177,14 +180,14 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
       TR(1);
       if (act) {
         // ---- S^T = K Q^T : s[gq][c] is the 32(kv) x 32(q) tile of kv chunk c ----
-        f32x16 s[QG][2];
+        f32x16 s[QG][KT];
 #pragma unroll
         for (int gq = 0; gq < QG; gq++)
 #pragma unroll
-          for (int c = 0; c < 2; c++)
+          for (int c = 0; c < KT; c++)
 #pragma unroll
             for (int r = 0; r < 16; r++) s[gq][c][r] = 0.f;
-        {
+        if constexpr (KT == 2) {
           V8 kf[2][C::KS];                                  // every K fragment of the tile is requested up front;
 #pragma unroll                                              // the MFMAs then start as the reads return in order
           for (int c = 0; c < 2; c++)
@@ -196,11 +199,20 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
             for (int t = 0; t < C::KS; t++)
 #pragma unroll
               for (int gq = 0; gq < QG; gq++) s[gq][c] = E::mfma(kf[c][t], qf[gq][t], s[gq][c]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < KT; c++)
+#pragma unroll
+            for (int t = 0; t < C::KS; t++) {
+              const V8 kf = lds_read_frag<T>(kbuf + koff[t] + c * 32 * C::PITCH);
+#pragma unroll
+              for (int gq = 0; gq < QG; gq++) s[gq][c] = E::mfma(kf, qf[gq][t], s[gq][c]);
+            }
         }
         TR(2);
         // element (gq, c, r): q = wq0 + 32 gq + l32 ; kv = kv0 + 32 c + 8 (r/4) + 4 g + r%4
-        const bool edge = apply_mask || (causal && (kv0 + 63 > wq0)) || (kv0 + 64 > a.Sk);
-        typename E::V8 pf[QG][2][2];
+        const bool edge = apply_mask || (causal && (kv0 + BN - 1 > wq0)) || (kv0 + BN > a.Sk);
+        typename E::V8 pf[QG][KT][2];
 #pragma unroll
         for (int gq = 0; gq < QG; gq++) {
           const int qrow = wq0 + 32 * gq + l32;
@@ -242,7 +254,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
           if (edge) {
             if (apply_mask) {
 #pragma unroll
-              for (int c = 0; c < 2; c++)
+              for (int c = 0; c < KT; c++)
 #pragma unroll
                 for (int r4 = 0; r4 < 4; r4++) {
                   const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
@@ -254,21 +266,21 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
                     if ((mbits >> (8 * e)) & 0xffu) s[gq][c][4 * r4 + e] += madd;
                 }
             }
-            if (causal && kv0 + 63 > wq0 + 32 * gq) {
+            if (causal && kv0 + BN - 1 > wq0 + 32 * gq) {
               // Keys after the query are removed outright: with the additive mask their probability
               // underflows to exactly 0 as well (the diagonal key is always visible), so the result
               // is the same bit for bit at a third of the vector instructions.
               const int dl = qrow - kv0 - 4 * g;
 #pragma unroll
-              for (int c = 0; c < 2; c++)
+              for (int c = 0; c < KT; c++)
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                   if (32 * c + 8 * (r >> 2) + (r & 3) > dl) s[gq][c][r] = -INFINITY;
             }
-            if (kv0 + 64 > a.Sk) {                             // ragged key tail
+            if (kv0 + BN > a.Sk) {                             // ragged key tail
               const int lim = a.Sk - kv0 - 4 * g;
 #pragma unroll
-              for (int c = 0; c < 2; c++)
+              for (int c = 0; c < KT; c++)
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                   if (32 * c + 8 * (r >> 2) + (r & 3) >= lim) s[gq][c][r] = -INFINITY;
@@ -277,7 +289,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
           // ---- online softmax for query row qrow ----
           float mx = s[gq][0][0];
 #pragma unroll
-          for (int c = 0; c < 2; c++)
+          for (int c = 0; c < KT; c++)
 #pragma unroll
             for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[gq][c][r]);
           mx = pair_max(mx);
@@ -291,9 +303,9 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
           const float mc = m_new * cmul;
           m[gq] = m_new;
           float rs = 0.f;
-          float p[2][16];
+          float p[KT][16];
 #pragma unroll
-          for (int c = 0; c < 2; c++)
+          for (int c = 0; c < KT; c++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
               p[c][r] = fast_exp2(__builtin_fmaf(s[gq][c][r], cmul, -mc));
@@ -302,9 +314,9 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
           lsum[gq] = lsum[gq] * alpha + rs;                  // row sum BEFORE dropout
           if (DROP) {
             // keep bits of this row and tile: word 2j + c covers keys 64j + 32c .. +31
-            const uint32_t* dr = a.droprow + ((int64_t)bh * a.Sq + qrow_c) * a.droprow_w + 2 * j;
+            const uint32_t* dr = a.droprow + ((int64_t)bh * a.Sq + qrow_c) * a.droprow_w + KT * j;
 #pragma unroll
-            for (int c = 0; c < 2; c++) {
+            for (int c = 0; c < KT; c++) {
               const uint32_t w = dr[c] >> (4 * g);
 #pragma unroll
               for (int r = 0; r < 16; r++) {
@@ -314,7 +326,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
             }
           }
 #pragma unroll
-          for (int c = 0; c < 2; c++)
+          for (int c = 0; c < KT; c++)
 #pragma unroll
             for (int hh = 0; hh < 2; hh++) {
               typename E::V2 t0 = E::cvt2(p[c][8 * hh + 0], p[c][8 * hh + 1]);
@@ -334,7 +346,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
         TR(3);
         // ---- O^T += V^T P^T ----
 #pragma unroll
-        for (int c = 0; c < 2; c++)
+        for (int c = 0; c < KT; c++)
 #pragma unroll
           for (int hh = 0; hh < 2; hh++)
 #pragma unroll
@@ -399,10 +411,16 @@ static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
   using C = SwzCfg<D>;
   constexpr int BM = 32 * QG * NW;
   a.n_tiles = (a.Sq + BM - 1) / BM;
-  constexpr size_t tiles = 4 * 64 * (size_t)C::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0), stage = (size_t)NW * 32 * (C::DB * 64 + 16);
-  const size_t smem = tiles > stage ? tiles : stage;
   const bool mask_t = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;
+  // The variants without any side input stream K/V in tiles of 128 keys where registers and LDS allow
+  // (8 waves x 32 rows, D <= 128): twice the matrix work between two barriers, -2 % (causal) to -6 % (full).
+  constexpr bool BIG = !BIAS && !DROP && QG == 1 && NW == 8 && D <= 128;
+  const int kt = (BIG && !mask_t) ? 4 : 2;
+  const size_t tiles = 4 * 32 * kt * (size_t)C::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0), stage = (size_t)NW * 32 * (C::DB * 64 + 16);
+  const size_t smem = tiles > stage ? tiles : stage;
   auto kern = mask_t ? fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, true> : fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, BIAS || DROP>;
+  if constexpr (BIG)
+    if (!mask_t) kern = fa_fwd_kernel<T, D, QG, NW, false, false, false, 4>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (e != hipSuccess) return e;
   const long long nblk = (long long)a.n_tiles * a.B * a.N;

@@ -569,8 +569,11 @@ def test_full_size_fa2_causal_fwd_bwd():
         sl = (slice(b, b + 1), slice(h, h + 1))
         _check_all(q[sl], k[sl], v[sl], dO[sl], dict(scale=scale, attn_mask=tri),
                    (o[sl], lse[sl], tuple(t[sl] for t in g)))
-    # the dense-mask path and the index-compare path agree (same blocks, same arithmetic)
-    assert torch.equal(o, oc) and all(torch.equal(a, b_) for a, b_ in zip(g, gc))
+    # the dense-mask path and the index-compare path agree: same blocks, same arithmetic up to the order of
+    # the online-softmax steps (the two paths stream keys in tiles of 64 and of 128), i.e. to an fp16 ulp
+    close = lambda x, y: torch.allclose(x.float(), y.float(), atol=1e-3, rtol=2e-3)
+    assert close(o, oc) and all(close(a, b_) for a, b_ in zip(g, gc))
+    assert torch.allclose(lse, lsec, atol=1e-5, rtol=1e-6)
     # linearity in V and in dO: O(v1 + v2) = O(v1) + O(v2), dV(2 dO) = 2 dV(dO)
     o2, _, g2 = _run(q, k, (v * 2).half(), (dO * 2).half(), scale=scale, mask_kind=_capi.MASK_CAUSAL, nxt=0)
     assert torch.allclose(o2.float(), 2 * oc.float(), atol=4e-3, rtol=2e-3)
