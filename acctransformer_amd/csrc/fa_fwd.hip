@@ -412,15 +412,13 @@ static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
   constexpr int BM = 32 * QG * NW;
   a.n_tiles = (a.Sq + BM - 1) / BM;
   const bool mask_t = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;
-  // The variants without any side input stream K/V in tiles of 128 keys where registers and LDS allow
+  // The variants without a bias stream K/V in tiles of 128 keys where registers and LDS allow
   // (8 waves x 32 rows, D <= 128): twice the matrix work between two barriers, -2 % (causal) to -6 % (full).
-  constexpr bool BIG = !BIAS && !DROP && QG == 1 && NW == 8 && D <= 128;
-  const int kt = (BIG && !mask_t) ? 4 : 2;
-  const size_t tiles = 4 * 32 * kt * (size_t)C::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0), stage = (size_t)NW * 32 * (C::DB * 64 + 16);
+  constexpr bool BIG = !BIAS && QG == 1 && NW == 8 && D <= 128;
+  constexpr int KT = BIG ? 4 : 2;
+  const size_t tiles = 4 * 32 * KT * (size_t)C::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0), stage = (size_t)NW * 32 * (C::DB * 64 + 16);
   const size_t smem = tiles > stage ? tiles : stage;
-  auto kern = mask_t ? fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, true> : fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, BIAS || DROP>;
-  if constexpr (BIG)
-    if (!mask_t) kern = fa_fwd_kernel<T, D, QG, NW, false, false, false, 4>;
+  auto kern = mask_t ? fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, true, KT> : fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, BIAS || DROP, KT>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (e != hipSuccess) return e;
   const long long nblk = (long long)a.n_tiles * a.B * a.N;
