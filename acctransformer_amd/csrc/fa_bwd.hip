@@ -162,12 +162,12 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
-    // block classes of a dense mask are fetched one tile ahead: the load has a whole tile to come back
+    // block classes of a dense mask: 64 blocks at a time into scalar registers
     const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
-    uint32_t fl_next = flrow ? flrow[j_lo >> 1] : 0u;
+    BlkClassWindow flwin;
+    flwin.init(flrow, 1, j_lo >> 1, j_hi >> 1, lane);
     for (int j = j_lo; j <= j_hi; j++) {
-      const uint32_t fl_cur = fl_next;
-      if (flrow && j < j_hi) fl_next = flrow[(j + 1) >> 1];
+      const uint32_t fl_cur = flwin.get(j >> 1, lane);
       const int buf = (j - j_lo) & 1;
       ACCT_LDS char* kbuf = smem + buf * 2 * TILEB;
       ACCT_LDS char* vbuf = kbuf + TILEB;
@@ -187,13 +187,15 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
       if (causal) act = act && (kv0 <= wq_end - 1);
       act = act && (kv0 < wkv_limit);
       bool apply_mask = false;
+      bool diag = causal;                                   // keys after the query are hidden, by index compare
       if (MASKT && a.mask_kind == kMaskDense && act) {
         act = fl_cur != kBlkSkip;
         apply_mask = fl_cur == kBlkApply;
+        if (fl_cur == kBlkTriu) { diag = true; act = kv0 <= wq_end - 1; }
       } else if (MASKT && a.mask_kind == kMaskTile) {
         apply_mask = wqb == kvb;
       }
-      const bool edge = apply_mask || (causal && (kv0 + 63 > wq0)) || (kv0 + 64 > a.Sk);
+      const bool edge = apply_mask || (diag && (kv0 + 63 > wq0)) || (kv0 + 64 > a.Sk);
       if (act) {
         V8 dsf[QG][2][2];
 #pragma unroll
@@ -234,7 +236,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
               // causal diagonal and/or ragged key tail only: P of a hidden key is exactly 0 (with the
               // additive mask it underflows to the same value), one compare and select per element
               int vis = a.Sk - 1 - kv0 - 32 * c - 4 * g;         // last visible key, relative to this lane's first
-              if (causal) vis = min(vis, qrow - kv0 - 32 * c - 4 * g);
+              if (diag) vis = min(vis, qrow - kv0 - 32 * c - 4 * g);
 #pragma unroll
               for (int r = 0; r < 16; r++) {
                 float p = fast_exp2(__builtin_fmaf(s[gq][r], a.scale_log2e, -lq[gq]));
@@ -281,10 +283,10 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
                     if ((mbits >> (8 * e)) & 0xffu) x[4 * r4 + e] += kMaskFill * kLog2e;
                 }
               }
-              if ((causal && (kv0 + 63 > wq0)) || (kv0 + 64 > a.Sk)) {
+              if ((diag && (kv0 + 63 > wq0)) || (kv0 + 64 > a.Sk)) {
                 // keys after the query (causal) or past Sk: P is exactly 0
                 int vis = a.Sk - 1 - kv0 - 32 * c - 4 * g;
-                if (causal) vis = min(vis, qrow - kv0 - 32 * c - 4 * g);
+                if (diag) vis = min(vis, qrow - kv0 - 32 * c - 4 * g);
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                   if (8 * (r >> 2) + (r & 3) > vis) x[r] = -INFINITY;
@@ -493,21 +495,26 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
                            (((uintptr_t)a.alibi & 15) | ((a.al_sb | a.al_sh | a.al_sq) & 7)) == 0;
   auto stage_bias = [&](int cn) { bias_tile_dma<T, false>(alibip, a.al_sq, cn * 32, a.Sq, wk0, a.Sk, bias_lds); };
 
-  // per-chunk predicates of this pair (chunk = 32 query rows; two per staged tile)
-  auto classify = [&](int cidx, uint32_t fl, bool& act, bool& apply_mask, bool& edge, bool& limits) {
+  // per-chunk predicates of this pair (chunk = 32 query rows; two per staged tile), as bits of one value
+  // so that they live in a register: 1 act, 2 apply_mask, 4 limits (some (row, key) of the chunk is
+  // absent), 8 diag (keys after the query are hidden, by index compare)
+  auto classify = [&](int cidx, uint32_t fl) -> uint32_t {
     const int qc0 = cidx * 32, qt0 = (cidx >> 1) * 64, qb = cidx >> 2;
-    act = (wkb - a.next_blk <= qb) && (qb <= wkb + a.prev_blk) && (wk0 < a.Sk);
+    bool act = (wkb - a.next_blk <= qb) && (qb <= wkb + a.prev_blk) && (wk0 < a.Sk);
     if (causal) act = act && (qt0 + 63 >= wk0);
     if (a.row_prefix) act = act && (wk0 < (qt0 / a.row_prefix + 1) * a.row_prefix);
-    apply_mask = false;
-    if (MASKT && a.mask_kind == kMaskDense && act) {
-      act = fl != kBlkSkip;                            // class of block (qb, wkb), fetched one step ahead
-      apply_mask = fl == kBlkApply;
+    bool apply_mask = false, diag = causal;
+    if (MASKT && a.mask_kind == kMaskDense) {
+      if (act) {
+        act = fl != kBlkSkip;                          // class of block (qb, wkb)
+        apply_mask = fl == kBlkApply;
+        if (fl == kBlkTriu) { diag = true; act = qt0 + 63 >= wk0; }
+      }
     } else if (MASKT && a.mask_kind == kMaskTile) {
       apply_mask = wkb == qb;
     }
-    limits = (causal && (wk0 + 63 > qc0)) || (wk0 + 64 > a.Sk) || (qc0 + 32 > a.Sq);   // some (row, key) of the chunk is absent
-    edge = BIAS || DROP || apply_mask || limits;
+    const bool limits = (diag && (wk0 + 63 > qc0)) || (wk0 + 64 > a.Sk) || (qc0 + 32 > a.Sq);
+    return (act ? 1u : 0u) | (apply_mask ? 2u : 0u) | (limits ? 4u : 0u) | (diag ? 8u : 0u);
   };
 
   if (i_lo <= i_hi) {
@@ -533,7 +540,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
       for (int db = 0; db < 2; db++) toff2_kept[db] = trow * C::PITCH + swz_off(4 * db + tchunk, C::swz(trow)) + 8 * (lane & 1);
     }
     const uint8_t* flcol = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + (int64_t)mb * a.Tr * a.Tc + wkb : nullptr;
-    uint32_t fl_next = flcol ? flcol[(int64_t)(c_lo >> 2) * a.Tc] : 0u;
+    BlkClassWindow flwin;
+    flwin.init(flcol, a.Tc, c_lo >> 2, c_hi >> 2, lane);
 #ifdef ACCT_TRACE
 #define TR(k) if (blockIdx.x == ACCT_TRACE && lane == 0 && n - c_lo < 96) ((unsigned long long*)((char*)a.delta + 2 * (size_t)a.B * a.N * a.Sq * 4))[((wave * 96) + (n - c_lo)) * 8 + (k)] = __builtin_amdgcn_s_memtime()
 #else
@@ -544,10 +552,9 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
       if ((n & 1) && (n >> 1) < i_hi) stage((n >> 1) + 1, smem + ((((n >> 1) + 1 - i_lo) & 1) * STAGEB));
       const int cidx = krole ? n - 1 : n;             // the chunk this wave works on in this step
       if (cidx >= c_lo && cidx <= c_hi) {
-        bool act, apply_mask, edge, limits;
-        const uint32_t fl_cur = fl_next;
-        if (flcol && cidx < c_hi) fl_next = flcol[(int64_t)((cidx + 1) >> 2) * a.Tc];
-        classify(cidx, fl_cur, act, apply_mask, edge, limits);
+        const uint32_t cls = classify(cidx, flwin.get(cidx >> 2, lane));
+        const bool act = cls & 1u, apply_mask = cls & 2u, limits = cls & 4u, diag = cls & 8u;
+        const bool edge = BIAS || DROP || apply_mask || limits;
         if (act) {
           const int c = cidx & 1, qc0 = cidx * 32;
           // Per-lane LDS offsets are re-derived in every step (a handful of VALU ops) rather than
@@ -665,7 +672,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 #pragma unroll
               for (int gk = 0; gk < 2; gk++) {
                 const int kv = wk0 + 32 * gk + l32;
-                int lo = causal ? kv - qc0 - 4 * g : -64;       // chunk rows below it come before the key
+                int lo = diag ? kv - qc0 - 4 * g : -64;         // chunk rows below it come before the key
                 int hi = a.Sq - 1 - qc0 - 4 * g;                // last query row that exists
                 if (kv >= a.Sk) hi = -64;
 #pragma unroll

@@ -132,7 +132,7 @@ struct FaArgs {
 };
 
 enum : int { kMaskNone = 0, kMaskDense = 1, kMaskTile = 3, kMaskCausal = 4 };
-enum : uint8_t { kBlkClean = 0, kBlkApply = 1, kBlkSkip = 2 };
+enum : uint8_t { kBlkClean = 0, kBlkApply = 1, kBlkSkip = 2, kBlkTriu = 3 };
 
 // Workgroup id -> (batch*head, launch rank of the tile; rank 0 is launched first).  Workgroups are
 // handed to the 8 XCDs round robin (id % 8), each XCD with its own L2.  With many heads the plain
@@ -170,6 +170,34 @@ ACCT_DEV void trim_dead_tiles(int& lo, int& hi, int lane, F dead) {
     hi -= 64;
   }
 }
+
+// Classes of 64 consecutive blocks of one row or column of the block-class table, as two 64-bit lane
+// masks in scalar registers: one byte load per lane and two ballots fill the window, and a step of the
+// tile loop then looks its block up with scalar shifts.  (A byte load per step would stall the step for
+// a round trip to memory, since the class decides a wave-uniform branch.)  Blocks are asked for in
+// ascending order; the window moves on when the block asked for lies past its end.
+struct BlkClassWindow {
+  const uint8_t* p;
+  int64_t stride;
+  int last, base;
+  uint64_t b0, b1;
+  ACCT_DEV void init(const uint8_t* p_, int64_t stride_, int first, int last_, int lane) {
+    p = p_; stride = stride_; last = last_;
+    load(first, lane);
+  }
+  ACCT_DEV void load(int first, int lane) {
+    base = first;
+    const int blk = first + lane;
+    const uint32_t f = (p && blk <= last) ? p[blk * stride] : 0u;
+    b0 = __ballot(f & 1u);
+    b1 = __ballot(f & 2u);
+  }
+  ACCT_DEV uint32_t get(int blk, int lane) {
+    if (blk - base >= 64) load(blk, lane);
+    const int sh = blk - base;
+    return (uint32_t)((b0 >> sh) & 1u) | ((uint32_t)((b1 >> sh) & 1u) << 1);
+  }
+};
 
 // four consecutive mask / dropout bytes starting at column kv of a row
 ACCT_DEV uint32_t load_u8x4(const uint8_t* row, int kv, int limit, bool vec_ok) {

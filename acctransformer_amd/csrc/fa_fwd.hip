@@ -145,13 +145,13 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
 #else
 #define TR(k)
 #endif
-    // block classes of a dense mask are fetched one tile ahead: the load has a whole tile to come back
+    // block classes of a dense mask: 64 blocks at a time into scalar registers
     const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
-    uint32_t fl_next = flrow ? flrow[j_lo / TPB] : 0u;
+    BlkClassWindow flwin;
+    flwin.init(flrow, 1, j_lo / TPB, j_hi / TPB, lane);
     for (int j = j_lo; j <= j_hi; j++) {
       TR(0);
-      const uint32_t fl_cur = fl_next;
-      if (flrow && j < j_hi) fl_next = flrow[(j + 1) / TPB];
+      const uint32_t fl_cur = flwin.get(j / TPB, lane);
       const int buf = (j - j_lo) & 1;
       ACCT_LDS char* kbuf = smem + buf * 2 * TILEB;
       ACCT_LDS char* vbuf = kbuf + TILEB;
@@ -171,9 +171,11 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
       if (causal) act = act && (kv0 <= wq_end - 1);
       act = act && (kv0 < wkv_limit);
       bool apply_mask = false;
+      bool diag = causal;                                   // keys after the query are hidden, by index compare
       if (MASKT && a.mask_kind == kMaskDense && act) {
         act = fl_cur != kBlkSkip;
         apply_mask = fl_cur == kBlkApply;
+        if (fl_cur == kBlkTriu) { diag = true; act = kv0 <= wq_end - 1; }
       } else if (MASKT && a.mask_kind == kMaskTile) {
         apply_mask = wqb == kvb;
       }
@@ -211,7 +213,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
         }
         TR(2);
         // element (gq, c, r): q = wq0 + 32 gq + l32 ; kv = kv0 + 32 c + 8 (r/4) + 4 g + r%4
-        const bool edge = apply_mask || (causal && (kv0 + BN - 1 > wq0)) || (kv0 + BN > a.Sk);
+        const bool edge = apply_mask || (diag && (kv0 + BN - 1 > wq0)) || (kv0 + BN > a.Sk);
         typename E::V8 pf[QG][KT][2];
 #pragma unroll
         for (int gq = 0; gq < QG; gq++) {
@@ -266,7 +268,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
                     if ((mbits >> (8 * e)) & 0xffu) s[gq][c][4 * r4 + e] += madd;
                 }
             }
-            if (causal && kv0 + BN - 1 > wq0 + 32 * gq) {
+            if (diag && kv0 + BN - 1 > wq0 + 32 * gq) {
               // Keys after the query are removed outright: with the additive mask their probability
               // underflows to exactly 0 as well (the diagonal key is always visible), so the result
               // is the same bit for bit at a third of the vector instructions.

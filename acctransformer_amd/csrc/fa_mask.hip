@@ -6,13 +6,16 @@
 // fp32 to every row that has at least one unmasked visible key elsewhere, and
 // can be skipped without changing a bit of the result; a block with no masked
 // entry needs no mask loads.  This pre-pass finds both kinds so the attention
-// kernels touch the mask only on mixed blocks.
+// kernels touch the mask only on mixed blocks.  A diagonal block (same 128 rows and keys) whose entries
+// are exactly "masked iff the key comes after the query" - every diagonal block of a causal mask given
+// as a tensor, with or without padding elsewhere - gets a class of its own: the kernels then compare
+// indices there, as they do for the causal mask kind, instead of loading mask bytes.
 #include "fa_common.hpp"
 #include "fa_launch.hpp"
 
 namespace acct {
 
-constexpr uint8_t kBlkAllMasked = 3;   // provisional: resolved to skip or apply below
+constexpr uint8_t kBlkAllMasked = 255;  // provisional: resolved to skip or apply below
 
 // Fast path (Sk and the mask pointers 16-byte aligned, at most 64 column blocks per pass): one
 // workgroup of 1024 threads per (mask batch, q block); thread t owns the 16-byte piece t%8 of row
@@ -30,6 +33,7 @@ __global__ void __launch_bounds__(1024) fa_mask_blocks_vec_kernel(const FaArgs a
   for (int kvb = tid; kvb < a.Tc; kvb += 1024)
     if (kvb < lo || kvb > hi) frow[kvb] = kBlkClean;
   bool row_unmasked = false;
+  bool tri_bad = false;                                 // the diagonal block differs from "key after query"
   for (int base = lo; base <= hi; base += 64) {        // 64 column blocks per pass
     if (tid == 0) { s_m = 0; s_u = 0; }
     __syncthreads();
@@ -50,6 +54,11 @@ __global__ void __launch_bounds__(1024) fa_mask_blocks_vec_kernel(const FaArgs a
           }
           if (has_nonzero) bm |= 1ull << i;
           if (has_zero) bu |= 1ull << i;
+          if (base + i == qb) {
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+              tri_bad |= (((v[e >> 2] >> (8 * (e & 3))) & 0xffu) != 0) != (c0 + e > (tid >> 3));
+          }
         }
       }
     }
@@ -73,8 +82,11 @@ __global__ void __launch_bounds__(1024) fa_mask_blocks_vec_kernel(const FaArgs a
   row_unmasked |= (bool)__shfl_xor((int)row_unmasked, 2);
   row_unmasked |= (bool)__shfl_xor((int)row_unmasked, 4);
   const int rows_ok = __syncthreads_and(row >= a.Sq || row_unmasked);
-  for (int kvb = lo + tid; kvb <= hi; kvb += 1024)
+  const int not_tri = __syncthreads_or(tri_bad);
+  for (int kvb = lo + tid; kvb <= hi; kvb += 1024) {
     if (frow[kvb] == kBlkAllMasked) frow[kvb] = rows_ok ? kBlkSkip : kBlkApply;
+    else if (kvb == qb && frow[kvb] == kBlkApply && !not_tri) frow[kvb] = kBlkTriu;
+  }
 }
 
 // Generic path (any alignment): one workgroup per (mask batch, q block); thread t scans 64 columns of row t/2
@@ -89,6 +101,7 @@ __global__ void __launch_bounds__(256) fa_mask_blocks_kernel(const FaArgs a, uin
   for (int kvb = tid; kvb < a.Tc; kvb += 256)
     if (kvb < lo || kvb > hi) frow[kvb] = kBlkClean;
   bool row_unmasked = false;
+  bool tri_bad = false;
   for (int kvb = lo; kvb <= hi; kvb++) {
     bool any_m = false, any_u = false;
     if (row < a.Sq) {
@@ -100,7 +113,11 @@ __global__ void __launch_bounds__(256) fa_mask_blocks_kernel(const FaArgs a, uin
         const uint32_t bits = load_u8x4(mrow, kv, a.Sk, vec_ok);
 #pragma unroll
         for (int e = 0; e < 4; e++)
-          if (e < n) { if ((bits >> (8 * e)) & 0xffu) any_m = true; else any_u = true; }
+          if (e < n) {
+            const bool masked = ((bits >> (8 * e)) & 0xffu) != 0;
+            if (masked) any_m = true; else any_u = true;
+            if (kvb == qb) tri_bad |= masked != (c0 + c + e > (tid >> 1));
+          }
       }
     }
     row_unmasked |= any_u;
@@ -110,8 +127,11 @@ __global__ void __launch_bounds__(256) fa_mask_blocks_kernel(const FaArgs a, uin
   row_unmasked |= (bool)__shfl_xor((int)row_unmasked, 1);
   const int rows_ok = __syncthreads_and(row >= a.Sq || row_unmasked);
   // (the barrier above also orders thread 0's provisional writes before the reads below)
-  for (int kvb = lo + tid; kvb <= hi; kvb += 256)
+  const int not_tri = __syncthreads_or(tri_bad);
+  for (int kvb = lo + tid; kvb <= hi; kvb += 256) {
     if (frow[kvb] == kBlkAllMasked) frow[kvb] = rows_ok ? kBlkSkip : kBlkApply;
+    else if (kvb == qb && frow[kvb] == kBlkApply && !not_tri) frow[kvb] = kBlkTriu;
+  }
 }
 
 // Column bitmaps of the mixed ('apply') blocks for the dK/dV kernel, whose lanes own key columns: one

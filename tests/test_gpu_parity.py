@@ -223,6 +223,46 @@ def test_ragged_dropout_with_random_mask(Sq, Sk):
                                       drop_mask=drop, keep_prob=0.8))
 
 
+@pytest.mark.parametrize("case", ["causal_padding", "ragged", "rectangular", "near_causal", "with_bias_dropout"])
+def test_dense_mask_with_causal_diagonal_blocks(case):
+    # A causal mask given as a tensor: its diagonal 128x128 blocks are recognised by the block pre-pass and
+    # handled by index compare; a block that differs from the pattern in one entry must fall back to the
+    # mask bytes.  Aligned and unaligned key lengths take different pre-pass kernels.
+    B, N, D = 3, 2, 128
+    Sq, Sk = {"causal_padding": (512, 512), "ragged": (333, 333), "rectangular": (300, 520),
+              "near_causal": (384, 384), "with_bias_dropout": (256, 256)}[case]
+    q, dO = (_gen((B, N, Sq, D), s) for s in (81, 84))
+    k, v = (_gen((B, N, Sk, D), s) for s in (82, 83))
+    rng = np.random.default_rng(85)
+    mask = np.broadcast_to(np.triu(np.ones((Sq, Sk), np.uint8), 1), (B, Sq, Sk)).copy()
+    if case == "causal_padding":
+        lens = np.array([130, 512, 300])
+        mask |= (np.arange(Sk)[None, None, :] >= lens[:, None, None]).astype(np.uint8)
+    elif case == "near_causal":
+        mask[0, 200, 131] = 1                            # one hidden key below the diagonal of block (1, 1)
+        mask[1, 140, 250] = 0                            # one visible key above it
+        mask[2, 383, 383] = 1                            # the last diagonal entry hidden (block (2, 2))
+    okw = dict(scale=D ** -0.5, attn_mask=mask)
+    kw = dict(mask_kind=_capi.MASK_DENSE_U8, attn_mask=mask)
+    if case == "with_bias_dropout":
+        # V at half scale: the first rows see one or two keys, where the exact dQ is 0 and the computed one is
+        # the fp16 rounding of O times dO.O / keep_prob, which at unit scale reaches the gate by itself
+        # (the same value on the index-compare path and on the mask-byte path)
+        v = (0.5 * v.float()).half()
+        drop = (rng.random((B, N, Sq, Sk)) < 0.85).astype(np.uint8)
+        al = (0.05 * torch.randn((1, N, Sq, Sk), generator=torch.Generator().manual_seed(86))).half()
+        okw.update(drop_mask=drop, keep_prob=0.85, alibi=al.float().numpy())
+        kw.update(drop_mask=drop, keep_prob=0.85, alibi=al)
+    res = _run(q, k, v, dO, scale=D ** -0.5, **kw)
+    _check_all(q, k, v, dO, okw, res)
+    if case in ("ragged", "rectangular"):
+        # the same mask by index compare from the start: the diagonal blocks take the same arithmetic
+        o2, lse2, g2 = _run(q, k, v, dO, scale=D ** -0.5, mask_kind=_capi.MASK_CAUSAL)
+        assert torch.allclose(res[0].float(), o2.float(), atol=1e-3, rtol=2e-3)
+        for a, b in zip(res[2], g2):
+            assert torch.allclose(a.float(), b.float(), atol=2e-3, rtol=2e-3)
+
+
 @pytest.mark.parametrize("dtype, Sq, Sk, D", [(torch.float16, 333, 328, 128), (torch.float16, 200, 333, 128),
                                               (torch.bfloat16, 300, 456, 128), (torch.float16, 260, 392, 80)])
 def test_all_side_inputs_ragged(dtype, Sq, Sk, D):
