@@ -115,6 +115,31 @@ def test_unequal_q_kv_lengths(q_len, kv_len):
     _check_all(q, k, v, dO, dict(scale=D ** -0.5), _run(q, k, v, dO, scale=D ** -0.5))
 
 
+@pytest.mark.parametrize("q_len, kv_len", [(256, 16500), (16500, 256)])
+def test_dense_mask_over_more_than_64_blocks(q_len, kv_len):
+    # The kernels hold the classes of 64 blocks of a mask row (forward, dQ) or column (dK/dV) at a time; here
+    # a row or column has 129 of them, of every class: wholly hidden, wholly visible, mixed, and (on the
+    # diagonal) the causal pattern.
+    D = 64
+    q, dO = _gen((1, 2, q_len, D), 91), _gen((1, 2, q_len, D), 94)
+    k, v = _gen((1, 2, kv_len, D), 92), _gen((1, 2, kv_len, D), 93)
+    rng = np.random.default_rng(95)
+    nqb, nkb = -(-q_len // 128), -(-kv_len // 128)
+    cls = rng.integers(0, 3, size=(nqb, nkb))            # 0 visible, 1 hidden, 2 mixed
+    mask = np.repeat(np.repeat((cls == 1).astype(np.uint8), 128, 0), 128, 1)[:q_len, :kv_len].copy()
+    mixed = (rng.random((q_len, kv_len)) < 0.5).astype(np.uint8)
+    sel = np.repeat(np.repeat(cls == 2, 128, 0), 128, 1)[:q_len, :kv_len]
+    mask[sel] = mixed[sel]
+    tri = np.triu(np.ones((128, 128), np.uint8), 1)
+    for d in range(min(nqb, nkb)):
+        blk = mask[128 * d:128 * d + 128, 128 * d:128 * d + 128]
+        blk[:] = tri[:blk.shape[0], :blk.shape[1]]
+    mask[:, 0] = 0                                       # every row keeps a visible key
+    mask = mask[None]
+    okw = dict(scale=D ** -0.5, attn_mask=mask)
+    _check_all(q, k, v, dO, okw, _run(q, k, v, dO, scale=D ** -0.5, mask_kind=_capi.MASK_DENSE_U8, attn_mask=mask))
+
+
 def test_reference_style_raw_op_inputs():
     # the reference drives the raw op (scale = 1) with uniform [0,1) inputs forward
     # (ST/test_fa_fwd_precision.py:23-25) and gates with data_compare (ST/common.py:178-192);
