@@ -153,10 +153,14 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
     for (int gq = 0; gq < QG; gq++)
       bias_tile_dma<T>(alibip, a.al_sq, wq0 + 32 * gq, a.Sq, jn * 64, a.Sk, bias_lds + gq * 4096);
   };
+  // keep bits of this wave's rows and one tile, staged with the tile's DMA (double buffered)
+  using DropStage = DropRowStage<DROP, QG, 2>;
+  ACCT_LDS char* drop_lds = smem + 4 * TILEB + (BIAS ? NW * QG * 4096 : 0) + wave * (2 * DropStage::BYTES);
   if (j_lo <= j_hi) {
     tile_dma<T, D, 64, NW>(kp, a.k_ss, j_lo * 64, a.Sk, smem);
     tile_dma<T, D, 64, NW>(vp, a.v_ss, j_lo * 64, a.Sk, smem + TILEB);
     if (BIAS && bias_staged && wq0 < a.Sq) stage_bias(j_lo);
+    DropStage::issue(a, bh, wq0, j_lo, lane, drop_lds);
     // A full wait the compiler can see: every load issued so far (Q, dO fragments included) is complete,
     // so it places no vmcnt wait inside the loop -- such a wait would also stall on the next tile's DMA.
     __builtin_amdgcn_s_waitcnt(0);
@@ -180,6 +184,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
           tile_dma<T, D, 64, NW>(kp, a.k_ss, (j + 1) * 64, a.Sk, nb);
           tile_dma<T, D, 64, NW>(vp, a.v_ss, (j + 1) * 64, a.Sk, nb + TILEB);
         }
+        DropStage::issue(a, bh, wq0, j + 1, lane, drop_lds + (buf ^ 1) * DropStage::BYTES);
       }
       const int kv0 = j * 64;
       const int kvb = j >> 1;
@@ -292,7 +297,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
                   if (8 * (r >> 2) + (r & 3) > vis) x[r] = -INFINITY;
               }
               uint32_t dw = 0xffffffffu;                        // keep bits of this row: keys kv0 + 32c .. +31
-              if (DROP) dw = a.droprow[((int64_t)bh * a.Sq + qrow_c) * a.droprow_w + 2 * j + c] >> (4 * g);
+              if (DROP) dw = DropStage::word(drop_lds + buf * DropStage::BYTES, 32 * gq + l32, c) >> (4 * g);
 #pragma unroll
               for (int r = 0; r < 16; r++) {
                 const float p = fast_exp2(x[r]);
@@ -374,11 +379,6 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 template <int D, bool BIAS, bool MASKT>
 constexpr int dkdv_park() { return D >= 128 ? (BIAS ? ACCT_PARK - 1 : (MASKT ? ACCT_PARK : ACCT_PARK_HOT)) : 0; }
 
-ACCT_DEV void dma4(const void* src, ACCT_LDS char* dst) {
-  const uint32_t d = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst);
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(d) : "memory");
-}
-
 // MASKT = false compiles the mask-tensor handling out (no mask, or the causal mask by index compare):
 // the hot variant must not carry that code's register pressure.
 template <typename T, int D, bool BIAS, bool DROP, bool MASKT>
@@ -390,7 +390,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   constexpr int BNK = 256;                          // key rows per workgroup
   constexpr int TILEB = 64 * C::PITCH;
   constexpr int STATB = 2 * 64 * 4;                 // -LSE*log2(e) and D of the 64 rows of a tile
-  constexpr int STAGEB = 2 * TILEB + STATB;         // one buffer: Q tile | dO tile | -LSE*log2(e) | D
+  constexpr int DROPB = DROP ? 2048 : 0;            // keep bits of the tile's 64 rows for the workgroup's 256 keys: [key][2 chunks] words
+  constexpr int STAGEB = 2 * TILEB + STATB + DROPB; // one buffer: Q tile | dO tile | -LSE*log2(e) | D | keep bits
   constexpr int PXB = 4096;                         // P of one pair and chunk: 64 lanes x 64 bytes
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 stage buffers][2 x 4 pair P buffers]
@@ -488,6 +489,14 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     if (wave < 2) {                                  // (pointers rebuilt from the kernel arguments: nothing to keep live)
       const int r = min(i * 64 + lane, a.Sq - 1);
       dma4((wave == 0 ? a.nlse : a.delta) + (int64_t)bh * a.Sq + r, sb + 2 * TILEB + wave * 256);
+    }
+    if (DROP) {
+      // word c of key k (LDS dword 2k + c) = rows 64i + 32c .. +31 of that key's column entry; one dword per lane.
+      // Read from LDS in the loop, the words cost no wait on the vector-memory counter, which would also wait
+      // for the tile DMA in flight.
+      const int idx = wave * 64 + lane, key = min(k0 + (idx >> 1), a.Sk - 1);
+      dma4(a.dropcol + ((((int64_t)bh * a.Tr + (i >> 1)) * a.Sk + key) << 2) + 2 * (i & 1) + (idx & 1),
+           sb + 2 * TILEB + STATB + wave * 256);
     }
   };
 
@@ -610,9 +619,9 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
           TR(1);
           uint32_t dcw[2] = {0u, 0u};                 // keep bits of the chunk's 32 rows for this lane's two key columns
           if (DROP) {
-            const uint32_t* dc = a.dropcol + ((((int64_t)bh * a.Tr + (qc0 >> 7)) * a.Sk) << 2) + ((qc0 >> 5) & 3);
+            const ACCT_LDS uint32_t* dc = (const ACCT_LDS uint32_t*)(qbuf + 2 * TILEB + STATB) + 2 * (pair * 64 + l32) + c;
 #pragma unroll
-            for (int gk = 0; gk < 2; gk++) dcw[gk] = dc[min(wk0 + 32 * gk + l32, a.Sk - 1) * 4] >> (4 * g);
+            for (int gk = 0; gk < 2; gk++) dcw[gk] = dc[64 * gk] >> (4 * g);
           }
           V8 bfr[2][2];                               // B fragments of the second product: P (V role) or dS (K role)
           if (!krole) {
@@ -794,7 +803,7 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
     constexpr int QG = 1, NW = 8;
     constexpr int BM = 32 * QG * NW;
     using CS = SwzCfg<D>;
-    constexpr size_t tiles = 4 * 64 * (size_t)CS::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0), stage = (size_t)NW * 32 * (CS::DB * 64 + 16);
+    constexpr size_t tiles = 4 * 64 * (size_t)CS::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0) + (size_t)NW * 2 * DropRowStage<DROP, QG, 2>::BYTES, stage = (size_t)NW * 32 * (CS::DB * 64 + 16);
     const size_t smem = tiles > stage ? tiles : stage;
     a.n_tiles = (a.Sq + BM - 1) / BM;
     const bool mask_q = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;
@@ -807,9 +816,10 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
   }
   if (stages & kStageDkDv) {
     using CS = SwzCfg<D>;
-    constexpr size_t stageb = 2 * 64 * (size_t)CS::PITCH + 512;
+    constexpr size_t stageb = 2 * 64 * (size_t)CS::PITCH + 512 + (DROP ? 2048 : 0);
     constexpr size_t loopb = 2 * stageb + 8 * 4096 + 8 * (size_t)dkdv_park<D, BIAS, true>() * 1024 + (BIAS ? 4 * 4096 : 0),
                      epib = (size_t)8 * 32 * (CS::DB * 64 + 16);
+    static_assert(loopb <= 160 * 1024 && epib <= 160 * 1024, "the workgroup's LDS must fit the CU's 160 KB");
     const size_t smem2 = loopb > epib ? loopb : epib;
     a.n_tiles = (a.Sk + 255) / 256;
     const bool mask_t = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;

@@ -412,6 +412,35 @@ ACCT_DEV typename Elem<T>::V4 bias_tile_read(const ACCT_LDS char* tile, int row,
 // all of this wave's direct-to-LDS loads have landed
 ACCT_DEV void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// one dword per lane from global memory to LDS at dst + 4 * lane (dst wave-uniform)
+ACCT_DEV void dma4(const void* src, ACCT_LDS char* dst) {
+  const uint32_t d = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(d) : "memory");
+}
+
+// Keep-bit words (dropout, packed by query row) of the 32*QG rows of a wave and the KT 32-key chunks of one
+// K/V tile, brought into a wave-private LDS buffer [row][KT] by DMA together with the tile.  Read from LDS
+// in the tile loop, they need no wait on the vector-memory counter, which would also wait for the K/V
+// tile in flight.
+template <bool DROP, int QG, int KT>
+struct DropRowStage {
+  static constexpr int BYTES = DROP ? QG * 32 * KT * 4 : 0;
+  static ACCT_DEV void issue(const FaArgs& a, int bh, int wq0, int j, int lane, ACCT_LDS char* buf) {
+    if constexpr (DROP) {
+#pragma unroll
+      for (int k = 0; k < QG * KT / 2; k++) {
+        const int idx = lane + 64 * k;
+        const int row = min(wq0 + idx / KT, a.Sq - 1), w = min(KT * j + idx % KT, a.droprow_w - 1);
+        dma4(a.droprow + ((int64_t)bh * a.Sq + row) * a.droprow_w + w, buf + k * 256);
+      }
+    }
+  }
+  static ACCT_DEV uint32_t word(const ACCT_LDS char* buf, int row, int c) {
+    return reinterpret_cast<const ACCT_LDS uint32_t*>(buf)[row * KT + c];
+  }
+};
+
+
 // byte offset of logical chunk `lc` in a row whose swz3(row) is `swz`
 ACCT_DEV int swz_off(int lc, int swz) { return (lc ^ swz) << 4; }
 

@@ -131,10 +131,14 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
     for (int gq = 0; gq < QG; gq++)
       bias_tile_dma<T>(alibip, a.al_sq, wq0 + 32 * gq, a.Sq, jn * 64, a.Sk, bias_lds + gq * 4096);
   };
+  // keep bits of this wave's rows and one tile, staged with the tile's DMA (double buffered)
+  using DropStage = DropRowStage<DROP, QG, KT>;
+  ACCT_LDS char* drop_lds = smem + 4 * TILEB + (BIAS ? NW * QG * 4096 : 0) + wave * (2 * DropStage::BYTES);
   if (j_lo <= j_hi) {
     tile_dma<T, D, BN, NW>(kp, a.k_ss, j_lo * BN, a.Sk, smem);
     tile_dma<T, D, BN, NW>(vp, a.v_ss, j_lo * BN, a.Sk, smem + TILEB);
     if (BIAS && bias_staged && wq0 < a.Sq) stage_bias(j_lo);
+    DropStage::issue(a, bh, wq0, j_lo, lane, drop_lds);
     // A full wait the compiler can see: every load issued so far (Q fragments included) is complete, so
     // it places no vmcnt wait inside the loop -- such a wait would also stall on the next tile's DMA.
     __builtin_amdgcn_s_waitcnt(0);
@@ -164,6 +168,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
           tile_dma<T, D, BN, NW>(kp, a.k_ss, (j + 1) * BN, a.Sk, nb);
           tile_dma<T, D, BN, NW>(vp, a.v_ss, (j + 1) * BN, a.Sk, nb + TILEB);
         }
+        DropStage::issue(a, bh, wq0, j + 1, lane, drop_lds + (buf ^ 1) * DropStage::BYTES);
       }
       const int kv0 = j * BN;
       const int kvb = j / TPB;
@@ -315,11 +320,10 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
             }
           lsum[gq] = lsum[gq] * alpha + rs;                  // row sum BEFORE dropout
           if (DROP) {
-            // keep bits of this row and tile: word 2j + c covers keys 64j + 32c .. +31
-            const uint32_t* dr = a.droprow + ((int64_t)bh * a.Sq + qrow_c) * a.droprow_w + KT * j;
+            // keep bits of this row and tile: word c covers keys kv0 + 32c .. +31
 #pragma unroll
             for (int c = 0; c < KT; c++) {
-              const uint32_t w = dr[c] >> (4 * g);
+              const uint32_t w = DropStage::word(drop_lds + buf * DropStage::BYTES, 32 * gq + l32, c) >> (4 * g);
 #pragma unroll
               for (int r = 0; r < 16; r++) {
                 const int32_t sel = (int32_t)(w << (31 - (8 * (r >> 2) + (r & 3)))) >> 31;   // keep ? ~0 : 0
@@ -418,7 +422,7 @@ static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
   // (8 waves x 32 rows, D <= 128): twice the matrix work between two barriers, -2 % (causal) to -6 % (full).
   constexpr bool BIG = !BIAS && QG == 1 && NW == 8 && D <= 128;
   constexpr int KT = BIG ? 4 : 2;
-  const size_t tiles = 4 * 32 * KT * (size_t)C::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0), stage = (size_t)NW * 32 * (C::DB * 64 + 16);
+  const size_t tiles = 4 * 32 * KT * (size_t)C::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0) + (size_t)NW * 2 * DropRowStage<DROP, QG, KT>::BYTES, stage = (size_t)NW * 32 * (C::DB * 64 + 16);
   const size_t smem = tiles > stage ? tiles : stage;
   auto kern = mask_t ? fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, true, KT> : fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, BIAS || DROP, KT>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);

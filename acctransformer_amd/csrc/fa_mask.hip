@@ -134,25 +134,23 @@ __global__ void __launch_bounds__(256) fa_mask_blocks_kernel(const FaArgs a, uin
   }
 }
 
-// Column bitmaps of the mixed ('apply') blocks for the dK/dV kernel, whose lanes own key columns: one
-// thread per key column packs the 128 rows of a block into 128 bits, so that the kernel reads one
-// 32-bit word per lane and 32-row chunk instead of 16 single bytes.
-__global__ void __launch_bounds__(128) fa_mask_colbits_kernel(const FaArgs a, const uint8_t* flags, uint32_t* out) {
+// Column bitmaps of the mixed ('apply') blocks for the dK/dV kernel, whose lanes own key columns: the 128
+// rows of a block packed into 128 bits per key column, so that the kernel reads one 32-bit word per lane
+// and 32-row chunk instead of 16 single bytes.  One thread per key column and word (32 rows): the loads
+// of a thread are independent, and 512 threads keep enough of them in flight.
+__global__ void __launch_bounds__(512) fa_mask_colbits_kernel(const FaArgs a, const uint8_t* flags, uint32_t* out) {
   const int kvb = blockIdx.x % a.Tc, qb = (blockIdx.x / a.Tc) % a.Tr, mb = blockIdx.x / (a.Tc * a.Tr);
   if (flags[((int64_t)mb * a.Tr + qb) * a.Tc + kvb] != kBlkApply) return;
-  const int kv = kvb * 128 + threadIdx.x;
+  const int kv = kvb * 128 + (threadIdx.x & 127), i = threadIdx.x >> 7;
   if (kv >= a.Sk) return;
   const uint8_t* col = a.mask + (int64_t)mb * a.mask_sb + kv;
-  uint32_t w[4] = {0u, 0u, 0u, 0u};
+  uint32_t w = 0u;
 #pragma unroll
-  for (int i = 0; i < 4; i++)
-#pragma unroll 8
-    for (int r = 0; r < 32; r++) {
-      const int row = qb * 128 + 32 * i + r;
-      if (row < a.Sq && col[(int64_t)row * a.Sk]) w[i] |= 1u << r;
-    }
-  u32x4 v = {w[0], w[1], w[2], w[3]};
-  *reinterpret_cast<u32x4*>(out + (((int64_t)mb * a.Tr + qb) * a.Sk + kv) * 4) = v;
+  for (int r = 0; r < 32; r++) {
+    const int row = qb * 128 + 32 * i + r;
+    if (row < a.Sq && col[(int64_t)row * a.Sk]) w |= 1u << r;
+  }
+  out[(((int64_t)mb * a.Tr + qb) * a.Sk + kv) * 4 + i] = w;
 }
 
 // the same for the compact 128x128 tile that is applied on diagonal blocks: out[key][4]
@@ -172,7 +170,7 @@ hipError_t launch_mask_colbits(const FaArgs& a, const uint8_t* flags, uint32_t* 
     hipLaunchKernelGGL(fa_mask_tilebits_kernel, dim3(1), dim3(128), 0, st, a.mask, out);
     return hipGetLastError();
   }
-  hipLaunchKernelGGL(fa_mask_colbits_kernel, dim3((unsigned)(MB * a.Tr * a.Tc)), dim3(128), 0, st, a, flags, out);
+  hipLaunchKernelGGL(fa_mask_colbits_kernel, dim3((unsigned)(MB * a.Tr * a.Tc)), dim3(512), 0, st, a, flags, out);
   return hipGetLastError();
 }
 
