@@ -301,9 +301,14 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 #pragma unroll
               for (int r = 0; r < 16; r++) {
                 const float p = fast_exp2(x[r]);
-                float dpv = dp[gq][r];
-                if (DROP) dpv = ((dw >> (8 * (r >> 2) + (r & 3))) & 1u) ? dpv * a.inv_keep : 0.f;
-                ds[r] = p * (dpv - dl[gq]);
+                if (DROP) {
+                  // dP of a dropped key is 0, of a kept one dP / keep_prob: a one-bit signed field extract gives
+                  // the all-ones / all-zeros mask, and the scaling rides on the FMA that subtracts D
+                  const float dpk = __uint_as_float(__float_as_uint(dp[gq][r]) & (uint32_t)__builtin_amdgcn_sbfe((int)dw, 8 * (r >> 2) + (r & 3), 1));
+                  ds[r] = p * __builtin_fmaf(dpk, a.inv_keep, -dl[gq]);
+                } else {
+                  ds[r] = p * (dp[gq][r] - dl[gq]);
+                }
               }
             }
             dsf[gq][c][0] = pack8<T>(ds);
@@ -704,7 +709,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
                   for (int e = 0; e < 4; e++) {
                     p[4 * r4 + e] = fast_exp2(__builtin_fmaf(t0[gk][8 * hh + 4 * r4 + e], a.scale_log2e, lv[e]));
                     pd[4 * r4 + e] = p[4 * r4 + e];
-                    if (DROP) pd[4 * r4 + e] = ((dcw[gk] >> (16 * hh + 8 * r4 + e)) & 1u) ? p[4 * r4 + e] * a.inv_keep : 0.f;
+                    // dropped: 0; kept: P (the 1 / keep_prob is applied to dV once, at the end)
+                    if (DROP) pd[4 * r4 + e] = __uint_as_float(__float_as_uint(p[4 * r4 + e]) & (uint32_t)__builtin_amdgcn_sbfe((int)dcw[gk], 16 * hh + 8 * r4 + e, 1));
                   }
                 }
                 bfr[gk][hh] = pack8<T>(pd);
@@ -726,9 +732,11 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 #pragma unroll
                   for (int e = 0; e < 4; e++) {
                     float dpv = t0[gk][8 * hh + 4 * r4 + e];
-                    if (DROP) dpv = ((dcw[gk] >> (16 * hh + 8 * r4 + e)) & 1u) ? dpv * a.inv_keep : 0.f;
+                    float dpd = dpv - dv4[e];
+                    // dropped: dP = 0; kept: dP / keep_prob, scaled by the FMA that subtracts D
+                    if (DROP) dpd = __builtin_fmaf(__uint_as_float(__float_as_uint(dpv) & (uint32_t)__builtin_amdgcn_sbfe((int)dcw[gk], 16 * hh + 8 * r4 + e, 1)), a.inv_keep, -dv4[e]);
                     // (an FMA with a zero addend keeps the fp16 -> fp32 conversion inside one mixed-precision instruction)
-                    ds[4 * r4 + e] = __builtin_fmaf((float)ph[4 * r4 + e], dpv - dv4[e], 0.0f);
+                    ds[4 * r4 + e] = __builtin_fmaf((float)ph[4 * r4 + e], dpd, 0.0f);
                   }
                 }
                 bfr[gk][hh] = pack8<T>(ds);
@@ -763,7 +771,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   // ---- epilogue: dV (V role) / scale * dK (K role), transposed through the wave's own LDS region ----
   T* outp = krole ? (T*)a.dk + b * a.k_sb + h * a.k_sh : (T*)a.dv + b * a.v_sb + h * a.v_sh;
   const int64_t oss = krole ? a.k_ss : a.v_ss;
-  const float oscale = krole ? a.scale : 1.0f;
+  const float oscale = krole ? a.scale : (DROP ? a.inv_keep : 1.0f);
   constexpr int OPITCH = C::DB * 64 + 16;
   ACCT_LDS char* obuf = smem + wave * (32 * OPITCH);
 #pragma unroll

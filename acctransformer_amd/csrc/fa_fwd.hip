@@ -326,8 +326,8 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
               const uint32_t w = DropStage::word(drop_lds + buf * DropStage::BYTES, 32 * gq + l32, c) >> (4 * g);
 #pragma unroll
               for (int r = 0; r < 16; r++) {
-                const int32_t sel = (int32_t)(w << (31 - (8 * (r >> 2) + (r & 3)))) >> 31;   // keep ? ~0 : 0
-                p[c][r] = __uint_as_float(__float_as_uint(p[c][r] * a.inv_keep) & (uint32_t)sel);
+                const int32_t sel = __builtin_amdgcn_sbfe((int)w, 8 * (r >> 2) + (r & 3), 1);   // keep ? ~0 : 0
+                p[c][r] = __uint_as_float(__float_as_uint(p[c][r]) & (uint32_t)sel);        // (1 / keep_prob: once, on O)
               }
             }
           }
@@ -385,7 +385,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   for (int gq = 0; gq < QG; gq++) {
     const int row = wq0 + 32 * gq + l32;
     const float l = pair_sum(lsum[gq]);
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    const float inv = l > 0.f ? (DROP ? a.inv_keep : 1.0f) / l : 0.f;
     if (row < a.Sq && g == 0) a.lse[(int64_t)bh * a.Sq + row] = l > 0.f ? m[gq] * mnat + __logf(l) : -INFINITY;
 #pragma unroll
     for (int db = 0; db < C::DB; db++)
