@@ -207,9 +207,22 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
         for (int c = 0; c < 2; c++) {
           f32x16 s[QG], dp[QG];
 #pragma unroll
-          for (int gq = 0; gq < QG; gq++)
+          for (int gq = 0; gq < QG; gq++) {
+            if (BIAS && bias_staged) {
+              // the bias enters as the initial value of the score accumulators (bias / scale, the MFMAs add
+              // q.k): nothing per score afterwards, no bias registers alive next to the scores
+              typename E::V4 bv[4];
 #pragma unroll
-            for (int r = 0; r < 16; r++) { s[gq][r] = 0.f; dp[gq][r] = 0.f; }
+              for (int r4 = 0; r4 < 4; r4++) bv[r4] = bias_tile_read<T>(bias_lds + gq * 4096, l32, 4 * c + r4, g);
+#pragma unroll
+              for (int r = 0; r < 16; r++) s[gq][r] = (float)bv[r >> 2][r & 3] * a.inv_scale;
+            } else {
+#pragma unroll
+              for (int r = 0; r < 16; r++) s[gq][r] = 0.f;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++) dp[gq][r] = 0.f;
+          }
           {
             V8 kf[C::KS], vf[C::KS];
 #pragma unroll
@@ -225,19 +238,26 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 #pragma unroll
               for (int gq = 0; gq < QG; gq++) dp[gq] = E::mfma(vf[t], dof[gq][t], dp[gq]);
           }
+          if (BIAS && bias_staged && c == 1) {
+            // the whole bias tile has been read and the reads consumed: its LDS region can take the next
+            // tile, which has the rest of this step to land (the end-of-step wait covers it)
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (j < j_hi) stage_bias(j + 1);
+          }
           // element (gq, r): q = wq0 + 32 gq + l32 ; kv = kv0 + 32 c + 8 (r/4) + 4 g + r%4
 #pragma unroll
           for (int gq = 0; gq < QG; gq++) {
             const int qrow = wq0 + 32 * gq + l32;
             const int qrow_c = min(qrow, a.Sq - 1);
             float ds[16];
-            if (!edge && !BIAS && !DROP) {                   // interior tile: no side inputs at all
+            const bool bias_pending = BIAS && !bias_staged;  // (a staged bias is already inside s)
+            if (!edge && !bias_pending && !DROP) {           // interior tile: no side inputs at all
 #pragma unroll
               for (int r = 0; r < 16; r++) {
                 const float p = fast_exp2(__builtin_fmaf(s[gq][r], a.scale_log2e, -lq[gq]));
                 ds[r] = p * (dp[gq][r] - dl[gq]);
               }
-            } else if (!apply_mask && !BIAS && !DROP) {
+            } else if (!apply_mask && !bias_pending && !DROP) {
               // causal diagonal and/or ragged key tail only: P of a hidden key is exactly 0 (with the
               // additive mask it underflows to the same value), one compare and select per element
               int vis = a.Sk - 1 - kv0 - 32 * c - 4 * g;         // last visible key, relative to this lane's first
@@ -253,27 +273,13 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
               float x[16];
 #pragma unroll
               for (int r = 0; r < 16; r++) x[r] = __builtin_fmaf(s[gq][r], a.scale_log2e, -lq[gq]);
-              if (BIAS) {
-                if (bias_staged) {
-                  typename E::V4 bv[4];
+              if (BIAS && !bias_staged) {                    // a bias the DMA cannot stage (alignment): direct loads
 #pragma unroll
-                  for (int r4 = 0; r4 < 4; r4++) bv[r4] = bias_tile_read<T>(bias_lds + gq * 4096, l32, 4 * c + r4, g);
-                  if (c == 1 && gq == QG - 1) {
-                    // the whole tile has been read: its LDS region can take the next tile, which has the
-                    // rest of this step to land (the end-of-step wait covers it)
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                    if (j < j_hi) stage_bias(j + 1);
-                  }
+                for (int r4 = 0; r4 < 4; r4++) {
+                  float bias[4];
+                  load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv0 + 32 * c + 8 * r4 + 4 * g, a.Sk, alibi_vec, bias);
 #pragma unroll
-                  for (int r = 0; r < 16; r++) x[r] = __builtin_fmaf((float)bv[r >> 2][r & 3], kLog2e, x[r]);
-                } else {
-#pragma unroll
-                  for (int r4 = 0; r4 < 4; r4++) {
-                    float bias[4];
-                    load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv0 + 32 * c + 8 * r4 + 4 * g, a.Sk, alibi_vec, bias);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) x[4 * r4 + e] = __builtin_fmaf(bias[e], kLog2e, x[4 * r4 + e]);
-                  }
+                  for (int e = 0; e < 4; e++) x[4 * r4 + e] = __builtin_fmaf(bias[e], kLog2e, x[4 * r4 + e]);
                 }
               }
               if (apply_mask) {
@@ -568,7 +574,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
       if (cidx >= c_lo && cidx <= c_hi) {
         const uint32_t cls = classify(cidx, flwin.get(cidx >> 2, lane));
         const bool act = cls & 1u, apply_mask = cls & 2u, limits = cls & 4u, diag = cls & 8u;
-        const bool edge = BIAS || DROP || apply_mask || limits;
+        const bool edge = (BIAS && !bias_staged) || apply_mask || limits;   // (a staged bias is already inside the scores)
         if (act) {
           const int c = cidx & 1, qc0 = cidx * 32;
           // Per-lane LDS offsets are re-derived in every step (a handful of VALU ops) rather than
@@ -597,10 +603,26 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
           ACCT_LDS char* px = pexch + ((cidx & 1) * 4 + pair) * PXB + ln * 16;
           // rows of this lane's C registers: q = qc0 + 8 (r/4) + 4 g + r%4 ; key = wk0 + 32 gk + l32
           f32x16 t0[2];                               // S (V role) or dP (K role) of the two key groups
+          if (BIAS && bias_staged) {
+            // V role: the bias enters as the initial value of the score accumulators (bias / scale, the MFMAs
+            // add q.k): no bias registers alive next to the scores.  Transposed reads of the row-major tile:
+            // each hands a lane the four consecutive rows 8i + 4g .. +3 of its key column (a 16-lane group
+            // covers 4 rows x 16 keys and supplies the addresses of that block's 8-byte pieces)
+            const ACCT_LDS char* bl = bias_lds + (4 * g + ((lane & 15) >> 2)) * 128 + ((lane >> 4) & 1) * 32 + (lane & 3) * 8;
 #pragma unroll
-          for (int gk = 0; gk < 2; gk++)
+            for (int gk = 0; gk < 2; gk++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) t0[gk][r] = 0.f;
+              for (int i = 0; i < 4; i++) {
+                const typename E::V4 bv = __builtin_bit_cast(typename E::V4, lds_read_tr(bl + i * 8 * 128 + gk * 64));
+#pragma unroll
+                for (int e = 0; e < 4; e++) t0[gk][4 * i + e] = (float)bv[e] * a.inv_scale;
+              }
+          } else {
+#pragma unroll
+            for (int gk = 0; gk < 2; gk++)
+#pragma unroll
+              for (int r = 0; r < 16; r++) t0[gk][r] = 0.f;
+          }
           {
             // software pipeline: the fragments of k-step t+1 are requested before the MFMAs of k-step t
             const ACCT_LDS char* abuf = (krole ? dobuf : qbuf) + c * 32 * C::PITCH;
@@ -622,6 +644,10 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
             }
           }
           TR(1);
+          if (BIAS && bias_staged) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // bias tile consumed: stage the next chunk's
+            if (n < c_hi) stage_bias(n + 1);
+          }
           uint32_t dcw[2] = {0u, 0u};                 // keep bits of the chunk's 32 rows for this lane's two key columns
           if (DROP) {
             const ACCT_LDS uint32_t* dc = (const ACCT_LDS uint32_t*)(qbuf + 2 * TILEB + STATB) + 2 * (pair * 64 + l32) + c;
@@ -632,25 +658,10 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
           if (!krole) {
             if (EDGE_PATH) {
               // Side inputs and range limits are folded into the raw scores in place, in three short
-              // passes that each keep few values live: + bias/scale; - 10000/scale where the mask bit of
+              // passes that each keep few values live: + bias/scale (unstaged bias only); - 10000/scale where the mask bit of
               // (row, key) is set; -inf where the key comes after the query (causal) or where the key
               // or the query row does not exist (the probability is exactly 0 either way).
-              if (BIAS && bias_staged) {
-                // transposed reads of the row-major tile: each hands a lane the four consecutive rows
-                // 8i + 4g .. +3 of its key column (a 16-lane group covers 4 rows x 16 keys and supplies the
-                // addresses of that block's 8-byte pieces)
-                const ACCT_LDS char* bl = bias_lds + (4 * g + ((lane & 15) >> 2)) * 128 + ((lane >> 4) & 1) * 32 + (lane & 3) * 8;
-#pragma unroll
-                for (int gk = 0; gk < 2; gk++)
-#pragma unroll
-                  for (int i = 0; i < 4; i++) {
-                    const typename E::V4 bv = __builtin_bit_cast(typename E::V4, lds_read_tr(bl + i * 8 * 128 + gk * 64));
-#pragma unroll
-                    for (int e = 0; e < 4; e++) t0[gk][4 * i + e] += (float)bv[e] * a.inv_scale;
-                  }
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // tile consumed: stage the next chunk's
-                if (n < c_hi) stage_bias(n + 1);
-              } else if (BIAS) {
+              if (BIAS && !bias_staged) {                   // a bias the DMA cannot stage (alignment): direct loads
                 const int qlast = a.Sq - 1 - qc0;               // last valid row, relative to the chunk
                 const T* brow0 = alibip + (int64_t)qc0 * a.al_sq;
 #pragma unroll
