@@ -570,7 +570,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     for (int n = c_lo; n <= c_hi + 1; n++) {
       TR(0);
       if ((n & 1) && (n >> 1) < i_hi) stage((n >> 1) + 1, smem + ((((n >> 1) + 1 - i_lo) & 1) * STAGEB));
-      const int cidx = krole ? n - 1 : n;             // the chunk this wave works on in this step
+      const int cidx = __builtin_amdgcn_readfirstlane(krole ? n - 1 : n);   // the chunk this wave works on in this step (wave-uniform: scalar)
       if (cidx >= c_lo && cidx <= c_hi) {
         const uint32_t cls = classify(cidx, flwin.get(cidx >> 2, lane));
         const bool act = cls & 1u, apply_mask = cls & 2u, limits = cls & 4u, diag = cls & 8u;
