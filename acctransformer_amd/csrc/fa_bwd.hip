@@ -409,7 +409,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   ACCT_LDS char* pexch = smem + 2 * STAGEB;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, g = lane >> 5;
-  const int pair = wave & 3;
+  const int pair = __builtin_amdgcn_readfirstlane(wave & 3);   // wave-uniform: the pair's key range stays in scalar registers
   const bool krole = wave >= 4;                     // false: V role (S, P, dV); true: K role (dP, dS, dK)
   const int BH = a.B * a.N;
   int bh, kt;                                       // causal: the first key tiles are the heaviest
@@ -559,6 +559,12 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 #pragma unroll
       for (int db = 0; db < 2; db++) toff2_kept[db] = trow * C::PITCH + swz_off(4 * db + tchunk, C::swz(trow)) + 8 * (lane & 1);
     }
+    constexpr bool KEEP_FOFF = !BIAS && !DROP && !MASKT;   // the plain variant has the registers for the row-major offsets too
+    int foff4_kept[4] = {0, 0, 0, 0};
+    if (KEEP_FOFF) {
+#pragma unroll
+      for (int t = 0; t < 4; t++) foff4_kept[t] = l32 * C::PITCH + swz_off(2 * t + g, C::swz(l32));
+    }
     const uint8_t* flcol = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + (int64_t)mb * a.Tr * a.Tc + wkb : nullptr;
     BlkClassWindow flwin;
     flwin.init(flcol, a.Tc, c_lo >> 2, c_hi >> 2, lane);
@@ -585,7 +591,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
           asm volatile("" : "+v"(ln));
           int foff4[4];                               // row-major fragment of k-step t: row l32, chunk 2t + g
 #pragma unroll
-          for (int t = 0; t < 4; t++) foff4[t] = (ln & 31) * C::PITCH + swz_off(2 * t + (ln >> 5), C::swz(ln & 31));
+          for (int t = 0; t < 4; t++) foff4[t] = KEEP_FOFF ? foff4_kept[t] : (ln & 31) * C::PITCH + swz_off(2 * t + (ln >> 5), C::swz(ln & 31));
           int toff2[2];
           if (KEEP_TOFF) {
             toff2[0] = toff2_kept[0];
