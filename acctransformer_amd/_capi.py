@@ -40,6 +40,7 @@ class AcctFaParams(ctypes.Structure):
         ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
         ("attn_mask", ctypes.c_void_p), ("drop_mask", ctypes.c_void_p), ("alibi", ctypes.c_void_p),
         ("drop_seed", ctypes.c_uint64), ("drop_offset", ctypes.c_uint32), ("drop_philox", ctypes.c_int32),
+        ("drop_bits", ctypes.c_void_p), ("drop_bits_filled", ctypes.c_int32), ("reserved0", ctypes.c_int32),
     ]
 
 
@@ -77,6 +78,8 @@ def load():
     lib.acct_fa_bwd_dkdv.restype = ctypes.c_int
     lib.acct_fa_fwd_workspace_bytes.argtypes = [P]
     lib.acct_fa_fwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.acct_fa_drop_bits_bytes.argtypes = [P]
+    lib.acct_fa_drop_bits_bytes.restype = ctypes.c_size_t
     lib.acct_fa_bwd_workspace_bytes.argtypes = [P]
     lib.acct_fa_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.acct_last_error.argtypes = []
@@ -188,6 +191,20 @@ def _workspace(nbytes, device):
     if nbytes == 0:
         return None
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def attach_drop_bits(p, device):
+    """Give `p` a buffer for the keep bits of its dropout mask, so that the forward call packs (or draws)
+    them once and the backward call of the same step reads them: set `p.drop_bits_filled = 1` after the
+    first call.  Returns the buffer (the caller keeps it alive), or None when `p` has no dropout."""
+    lib = load()
+    n = lib.acct_fa_drop_bits_bytes(ctypes.byref(p))
+    if n == 0:
+        return None
+    buf = torch.empty(n, dtype=torch.uint8, device=device)
+    p.drop_bits = buf.data_ptr()
+    p.drop_bits_filled = 0
+    return buf
 
 
 def fa_fwd(p, q):

@@ -96,6 +96,7 @@ int validate(const acct_fa_params* p, bool backward) {
     if ((uintptr_t)ptrs[i] & 15) return fail(ACCT_E_SHAPE, "q, k and v must be 16-byte aligned");
   if (p->alibi && (p->alibi_stride_b < 0 || p->alibi_stride_h < 0 || p->alibi_stride_q < 0))
     return fail(ACCT_E_SHAPE, "alibi strides must be >= 0");
+  if ((uintptr_t)p->drop_bits & 255) return fail(ACCT_E_WORKSPACE, "drop_bits must be 256-byte aligned");
   return ACCT_OK;
 }
 
@@ -183,13 +184,19 @@ int acct_build_is_complete(void) { return acct::launch_variants_complete() ? 1 :
 
 size_t acct_fa_fwd_workspace_bytes(const acct_fa_params* p) {
   if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0 || p->Sk <= 0) return 0;
-  return flag_bytes(p) + droprow_bytes(p);
+  return flag_bytes(p) + (p->drop_bits ? 0 : droprow_bytes(p));
+}
+
+size_t acct_fa_drop_bits_bytes(const acct_fa_params* p) {
+  if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0 || p->Sk <= 0) return 0;
+  return droprow_bytes(p) + dropcol_bytes(p);
 }
 
 size_t acct_fa_bwd_workspace_bytes(const acct_fa_params* p) {
   if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0) return 0;
   if (p->Sk <= 0) return 0;
-  return 2 * align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + flag_bytes(p) + colbit_bytes(p) + droprow_bytes(p) + dropcol_bytes(p);
+  return 2 * align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + flag_bytes(p) + colbit_bytes(p) +
+         (p->drop_bits ? 0 : droprow_bytes(p) + dropcol_bytes(p));
 }
 
 int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, size_t workspace_bytes, void* stream) {
@@ -213,11 +220,15 @@ int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, s
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
   }
   if (dropout_on(p)) {
-    uint32_t* rows = (uint32_t*)((char*)workspace + flag_bytes(p));
+    // own bits by query row in the workspace, or both layouts in the caller's buffer for the backward call
+    uint32_t* rows = p->drop_bits ? (uint32_t*)p->drop_bits : (uint32_t*)((char*)workspace + flag_bytes(p));
+    uint32_t* cols = p->drop_bits ? (uint32_t*)((char*)p->drop_bits + droprow_bytes(p)) : nullptr;
     a.droprow = rows;
     a.droprow_w = (int)droprow_words(p);
-    hipError_t e = philox_on(p) ? acct::launch_drop_philox(a, rows, nullptr, st) : acct::launch_drop_bits(a, rows, nullptr, st);
-    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "dropout bitmap kernel: %s", hipGetErrorString(e));
+    if (!(p->drop_bits && p->drop_bits_filled)) {
+      hipError_t e = philox_on(p) ? acct::launch_drop_philox(a, rows, cols, st) : acct::launch_drop_bits(a, rows, cols, st);
+      if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "dropout bitmap kernel: %s", hipGetErrorString(e));
+    }
   }
   // 8 waves x 32 query rows (two waves per SIMD overlap MFMA and softmax work) once that still
   // fills the chip, else 4 waves x 32 rows for more workgroups
@@ -267,15 +278,23 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask bitmap kernel: %s", hipGetErrorString(e));
   }
   if (dropout_on(p)) {
-    char* base = (char*)workspace + 2 * stat_bytes + flag_bytes(p) + colbit_bytes(p);
+    char* base = p->drop_bits ? (char*)p->drop_bits : (char*)workspace + 2 * stat_bytes + flag_bytes(p) + colbit_bytes(p);
     uint32_t* rows = (uint32_t*)base;
     uint32_t* cols = (uint32_t*)(base + droprow_bytes(p));
     a.droprow = rows;
     a.dropcol = cols;
     a.droprow_w = (int)droprow_words(p);
-    hipError_t e = philox_on(p) ? acct::launch_drop_philox(a, want_dq ? rows : nullptr, want_dkdv ? cols : nullptr, st)
-                                : acct::launch_drop_bits(a, want_dq ? rows : nullptr, want_dkdv ? cols : nullptr, st);
-    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "dropout bitmap kernel: %s", hipGetErrorString(e));
+    if (p->drop_bits && p->drop_bits_filled) {
+      // an earlier call of this step left both layouts in the caller's buffer
+    } else if (p->drop_bits) {
+      // the caller's buffer is filled completely, whichever half of the backward asked
+      hipError_t e = philox_on(p) ? acct::launch_drop_philox(a, rows, cols, st) : acct::launch_drop_bits(a, rows, cols, st);
+      if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "dropout bitmap kernel: %s", hipGetErrorString(e));
+    } else {
+      hipError_t e = philox_on(p) ? acct::launch_drop_philox(a, want_dq ? rows : nullptr, want_dkdv ? cols : nullptr, st)
+                                  : acct::launch_drop_bits(a, want_dq ? rows : nullptr, want_dkdv ? cols : nullptr, st);
+      if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "dropout bitmap kernel: %s", hipGetErrorString(e));
+    }
   }
   hipError_t e = acct::launch_bwd(a, p->dtype, p->D, stages, st);
   if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "backward kernels: %s", hipGetErrorString(e));

@@ -147,7 +147,12 @@ class _FlashAttentionFn(torch.autograd.Function):
         q, k, v = _rows_contiguous(q), _rows_contiguous(k), _rows_contiguous(v)
         p = _build_params(q, k, v, attn_mask, dropout_mask, alibi_mask, prev_block_num, next_block_num, scale, keep_prob,
                           row_block_prefix)
+        # with dropout, the keep bits the forward packs (or draws) are kept for the backward of this step
+        needs_grad = any(ctx.needs_input_grad[:3])
+        ctx.drop_bits = _capi.attach_drop_bits(p, q.device) if needs_grad else None
         o, lse = _capi.fa_fwd(p, q)
+        if ctx.drop_bits is not None:
+            p.drop_bits_filled = 1
         ctx.save_for_backward(q, k, v, o, lse)
         ctx.params = p
         ctx.mark_non_differentiable(lse)

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define ACCT_FA_VERSION 102
+#define ACCT_FA_VERSION 103
 
 /* error codes (0 = success) */
 #define ACCT_OK          0
@@ -101,6 +101,18 @@ typedef struct acct_fa_params {
   uint64_t drop_seed;
   uint32_t drop_offset;
   int32_t  drop_philox;
+  /* Keep bits shared between the forward and the backward call of one training step (fields added in
+     version 103; no counterpart in the reference, whose two operators each read the byte mask).  Both
+     calls need the dropout mask as bit maps, packed from drop_mask or drawn from (drop_seed, drop_offset)
+     by a pre-pass.  With drop_bits == NULL every call runs that pre-pass into its own workspace.  With
+     drop_bits pointing at acct_fa_drop_bits_bytes(p) bytes of device memory (256-byte aligned) that the
+     caller keeps from the forward to the backward call, a call with drop_bits_filled == 0 runs the pre-pass
+     into that buffer and a call with drop_bits_filled != 0 reads what an earlier call left there.  The
+     caller sets drop_bits_filled after the first call returns; the bits depend on drop_mask or on
+     (drop_seed, drop_offset, keep_prob) and on B, N, Sq, Sk only. */
+  void*    drop_bits;
+  int32_t  drop_bits_filled;
+  int32_t  reserved0;
 } acct_fa_params;
 
 /* Forward: replaces the `flash_attention` TBE custom op, T/flash_attention_fwd.py:498-530
@@ -111,6 +123,9 @@ typedef struct acct_fa_params {
 int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE,
                 void* workspace, size_t workspace_bytes, void* stream);
 size_t acct_fa_fwd_workspace_bytes(const acct_fa_params* p);
+/* Size of the optional drop_bits buffer (0 without dropout): keep bits by query row for the forward and dQ
+ * kernels, then by key column for the dK/dV kernel, a quarter of a byte per score in total. */
+size_t acct_fa_drop_bits_bytes(const acct_fa_params* p);
 
 /* Backward: replaces the `flash_attention_grad` TBE custom op,
  * T/flash_attention_bwd.py:436-477 (the bprop of T/flash_attention_impl.py:117-124

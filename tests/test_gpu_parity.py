@@ -422,6 +422,64 @@ def test_flash_attention_layer_autograd():
         _gate(ref, got)
 
 
+@pytest.mark.parametrize("source", ["byte_mask", "seed_pair"])
+def test_keep_bits_shared_between_forward_and_backward(source):
+    # The forward call packs (or draws) the keep bits into a buffer the caller holds; the backward call of the
+    # same step reads them.  Every result equals, bit for bit, that of calls that each build their own bits; a
+    # backward that fills the buffer itself, and its two halves run separately on the filled buffer, agree too.
+    B, N, Sq, Sk, D = 2, 3, 300, 392, 128
+    q, dO = (_gen((B, N, Sq, D), s).to(DEV) for s in (101, 104))
+    k, v = (_gen((B, N, Sk, D), s).to(DEV) for s in (102, 103))
+    kw = dict(scale=D ** -0.5, keep_prob=0.8, mask_kind=_capi.MASK_CAUSAL)
+    if source == "byte_mask":
+        g = torch.Generator().manual_seed(105)
+        kw["drop_mask"] = (torch.rand((B, N, Sq, Sk), generator=g) < 0.8).to(torch.uint8).to(DEV)
+    else:
+        kw.update(drop_seed=0x1234567890ABCDEF, drop_offset=9)
+    p0 = _capi.make_params(q, k, v, **kw)
+    o0, lse0 = _capi.fa_fwd(p0, q)
+    g0 = _capi.fa_bwd(p0, q, k, v, o0, dO, lse0)
+
+    p1 = _capi.make_params(q, k, v, **kw)
+    bits = _capi.attach_drop_bits(p1, q.device)
+    assert bits is not None and bits.numel() == _capi.load().acct_fa_drop_bits_bytes(ctypes.byref(p1))
+    bits.fill_(0xA5)                                       # whatever was there before is overwritten
+    o1, lse1 = _capi.fa_fwd(p1, q)
+    p1.drop_bits_filled = 1
+    snapshot = bits.clone()
+    g1 = _capi.fa_bwd(p1, q, k, v, o1, dO, lse1)
+    assert torch.equal(bits, snapshot)                     # a filled buffer is only read
+    assert torch.equal(o0, o1) and torch.equal(lse0, lse1)
+    for a, b in zip(g0, g1):
+        assert torch.equal(a, b)
+
+    p2 = _capi.make_params(q, k, v, **kw)                  # backward first: it fills the buffer completely
+    bits2 = _capi.attach_drop_bits(p2, q.device)
+    g2 = _capi.fa_bwd(p2, q, k, v, o0, dO, lse0)
+    assert bits2 is not None
+    for a, b in zip(g0, g2):
+        assert torch.equal(a, b)
+
+
+def test_autograd_function_keeps_the_keep_bits_for_backward():
+    B, N, S, D = 1, 2, 256, 64
+    q, k, v, dO = (_gen((B, N, S, D), s).to(DEV) for s in (106, 107, 108, 109))
+    fa = get_flash_attention(scale=D ** -0.5, keep_prob=0.75)
+    res = []
+    for requires_grad in (True, False):
+        qd = q.clone().requires_grad_(requires_grad)
+        o, _ = fa(qd, k, v, None, (77, 3))
+        if requires_grad:
+            node = o.grad_fn
+            assert node.drop_bits is not None and node.params.drop_bits_filled == 1
+            o.backward(dO)
+            # the operator's own bprop closure builds its bits again and must agree
+            dq2 = fa.bprop(q, k, v, None, (77, 3), None, (o.detach(), _), (dO,))[0]
+            assert torch.equal(qd.grad, dq2)
+        res.append(o.detach())
+    assert torch.equal(res[0], res[1])                     # without gradients nothing is kept, same output
+
+
 def test_layer_dropout_uses_one_mask_forward_and_backward():
     B, N, S, D = 1, 2, 256, 64
     layer = FlashAttention(head_dim=D, dropout_rate=0.5).train()

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     decl = re.findall(r"^\s*(?:int|size_t|const char\*)\s+(acct_\w+)\s*\(", _header(), flags=re.M)
     assert set(decl) >= {"acct_fa_fwd", "acct_fa_bwd", "acct_fa_bwd_dq", "acct_fa_bwd_dkdv",
                          "acct_fa_fwd_workspace_bytes", "acct_fa_bwd_workspace_bytes", "acct_last_error", "acct_version",
-                         "acct_fa_infer_shape", "acct_build_is_complete"}
+                         "acct_fa_infer_shape", "acct_build_is_complete", "acct_fa_drop_bits_bytes"}
     for name in decl:
         assert hasattr(lib, name), name
     m = re.search(r"#define ACCT_FA_VERSION (\d+)", _header())
@@ -49,7 +49,7 @@ def test_struct_mirror_matches_header_field_order():
         for part in decl.split(","):
             names.append(re.sub(r"\[\d+\]", "", part.strip().split()[-1]).lstrip("*"))
     assert names == [f[0] for f in _capi.AcctFaParams._fields_]
-    assert ctypes.sizeof(_capi.AcctFaParams) == 240
+    assert ctypes.sizeof(_capi.AcctFaParams) == 256
 
 
 def _params(**over):
@@ -237,6 +237,28 @@ def test_counter_based_dropout_fields_and_workspace():
     with pytest.raises(ValueError):
         _capi.make_params(q, q.clone(), q.clone(), scale=1.0, keep_prob=0.9, drop_seed=1,
                           drop_mask=torch.ones(2, 2, 128, 128, dtype=torch.uint8))
+
+
+def test_shared_keep_bits_buffer_sizes_and_alignment():
+    lib = _capi.load()
+    assert lib.acct_version() >= 103
+    q = torch.zeros(2, 2, 128, 128, dtype=torch.float16)
+    p = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, keep_prob=0.9, drop_seed=3)
+    rows, cols = 2 * 2 * 128 * 4 * 4, 2 * 2 * 1 * 128 * 16
+    assert lib.acct_fa_drop_bits_bytes(ctypes.byref(p)) == rows + cols
+    stats = 2 * (2 * 2 * 128 * 4)
+    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p)) == stats + rows + cols
+    # with the caller's buffer attached, the calls no longer ask for room of their own for the bits
+    p.drop_bits = 256 * 1000
+    assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p)) == 0
+    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p)) == stats
+    # the buffer must be 256-byte aligned (checked before anything is launched)
+    p.drop_bits = 256 * 1000 + 16
+    buf = (ctypes.c_char * 64)()
+    assert lib.acct_fa_fwd(ctypes.byref(p), ctypes.addressof(buf), ctypes.addressof(buf), None, 0, None) == -7
+    # no dropout: nothing to share
+    p0 = _capi.make_params(q, q.clone(), q.clone(), scale=1.0)
+    assert lib.acct_fa_drop_bits_bytes(ctypes.byref(p0)) == 0
 
 
 # ---- the oracle still reproduces the committed fixtures -------------------------
