@@ -550,8 +550,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     // nothing is carried across it in registers.
     const int c_lo = 2 * i_lo, c_hi = 2 * i_hi + 1;
     // offsets of the transposed fragments of d block db: kept across the steps where the registers allow
-    // (a fifth of the step's vector instructions otherwise), re-derived in every step in the bias variants
-    constexpr bool KEEP_TOFF = !BIAS;
+    // (a fifth of the step's vector instructions otherwise), re-derived in every step in the bias + dropout variant
+    constexpr bool KEEP_TOFF = !(BIAS && DROP);
     int toff2_kept[2] = {0, 0};
     if (KEEP_TOFF) {
       const int trow = 4 * g + ((lane & 15) >> 2);
@@ -559,7 +559,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 #pragma unroll
       for (int db = 0; db < 2; db++) toff2_kept[db] = trow * C::PITCH + swz_off(4 * db + tchunk, C::swz(trow)) + 8 * (lane & 1);
     }
-    constexpr bool KEEP_FOFF = !BIAS && !DROP && !MASKT;   // the plain variant has the registers for the row-major offsets too
+    constexpr bool KEEP_FOFF = !BIAS;   // the variants without a bias have the registers for the row-major offsets too
     int foff4_kept[4] = {0, 0, 0, 0};
     if (KEEP_FOFF) {
 #pragma unroll
@@ -583,8 +583,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
         const bool edge = (BIAS && !bias_staged) || apply_mask || limits;   // (a staged bias is already inside the scores)
         if (act) {
           const int c = cidx & 1, qc0 = cidx * 32;
-          // Per-lane LDS offsets are re-derived in every step (a handful of VALU ops) rather than
-          // kept in registers.  Chunk c + 8 of a row sits in slot (c ^ swz) ^ 8: the row-major
+          // Where the registers do not allow keeping them (see above), the per-lane LDS offsets are
+          // re-derived in every step (a handful of VALU ops).  Chunk c + 8 of a row sits in slot (c ^ swz) ^ 8: the row-major
           // fragments of the upper half of the head dim are one XOR away from the lower four, and the
           // transposed ones (row % 16 < 8, swizzle bit 3 clear) 128 bytes after them.
           int ln = lane;
