@@ -15,7 +15,8 @@ _LIB_NAME = "libacct_fa.so"
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
 
 ACCT_F16, ACCT_BF16 = 0, 1
-MASK_NONE, MASK_DENSE_U8, MASK_TILE_U8, MASK_CAUSAL = 0, 1, 3, 4
+MASK_NONE, MASK_DENSE_U8, MASK_DENSE_F16, MASK_TILE_U8, MASK_CAUSAL, MASK_TILE_F16 = 0, 1, 2, 3, 4, 5
+DROP_U8, DROP_F16 = 0, 1
 BLOCK_UNBOUNDED = 65536
 
 ERROR_NAMES = {
@@ -40,7 +41,7 @@ class AcctFaParams(ctypes.Structure):
         ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
         ("attn_mask", ctypes.c_void_p), ("drop_mask", ctypes.c_void_p), ("alibi", ctypes.c_void_p),
         ("drop_seed", ctypes.c_uint64), ("drop_offset", ctypes.c_uint32), ("drop_philox", ctypes.c_int32),
-        ("drop_bits", ctypes.c_void_p), ("drop_bits_filled", ctypes.c_int32), ("reserved0", ctypes.c_int32),
+        ("drop_bits", ctypes.c_void_p), ("drop_bits_filled", ctypes.c_int32), ("drop_mask_kind", ctypes.c_int32),
     ]
 
 
@@ -115,9 +116,11 @@ def make_params(q, k, v, *, scale, keep_prob=1.0, prev_block_num=BLOCK_UNBOUNDED
                 mask_kind=MASK_NONE, attn_mask=None, drop_mask=None, alibi=None, o_like=None, row_block_prefix=0,
                 drop_seed=None, drop_offset=0):
     """Describe one attention problem.  q [B,N,Sq,D]; k,v [B,N,Sk,D] (any
-    batch/head/row strides, unit stride along D); attn_mask uint8 [1|B,Sq,Sk]
-    (DENSE) or [128,128] (TILE); drop_mask uint8 [B,N,Sq,Sk]; alibi in q's
-    dtype, broadcastable to [B,N,Sq,Sk].  With drop_seed (and no drop_mask) and
+    batch/head/row strides, unit stride along D); attn_mask [1|B,Sq,Sk]
+    (DENSE) or [128,128] (TILE), uint8 for the _U8 kinds and q's dtype for the
+    _F16 kinds (nonzero = masked); drop_mask [B,N,Sq,Sk], uint8 {0,1} or q's
+    dtype {0, 1/keep_prob} (nonzero = keep); alibi in q's dtype, broadcastable
+    to [B,N,Sq,Sk].  With drop_seed (and no drop_mask) and
     keep_prob < 1 the library draws the keep mask itself from
     (drop_seed, drop_offset), identically in forward and backward."""
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
@@ -146,10 +149,11 @@ def make_params(q, k, v, *, scale, keep_prob=1.0, prev_block_num=BLOCK_UNBOUNDED
         p.o_stride = _bhs_strides(o_like)
     p.q, p.k, p.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
     keep = [q, k, v]
-    if mask_kind in (MASK_DENSE_U8, MASK_TILE_U8):
-        if attn_mask is None or attn_mask.dtype != torch.uint8 or not attn_mask.is_contiguous():
-            raise TypeError("attn_mask must be a contiguous uint8 tensor")
-        if mask_kind == MASK_DENSE_U8:
+    if mask_kind in (MASK_DENSE_U8, MASK_TILE_U8, MASK_DENSE_F16, MASK_TILE_F16):
+        want = torch.uint8 if mask_kind in (MASK_DENSE_U8, MASK_TILE_U8) else q.dtype
+        if attn_mask is None or attn_mask.dtype != want or not attn_mask.is_contiguous():
+            raise TypeError(f"attn_mask must be a contiguous {want} tensor for mask_kind {mask_kind}")
+        if mask_kind in (MASK_DENSE_U8, MASK_DENSE_F16):
             if attn_mask.dim() != 3 or attn_mask.shape[1:] != (Sq, Sk) or attn_mask.shape[0] not in (1, B):
                 raise ValueError(f"attn_mask must be [1|B,{Sq},{Sk}], got {tuple(attn_mask.shape)}")
             p.mask_stride_b = 0 if attn_mask.shape[0] == 1 else Sq * Sk
@@ -158,9 +162,10 @@ def make_params(q, k, v, *, scale, keep_prob=1.0, prev_block_num=BLOCK_UNBOUNDED
         p.attn_mask = attn_mask.data_ptr()
         keep.append(attn_mask)
     if drop_mask is not None:
-        if drop_mask.dtype != torch.uint8 or not drop_mask.is_contiguous() or drop_mask.shape != (B, N, Sq, Sk):
-            raise TypeError(f"drop_mask must be contiguous uint8 [{B},{N},{Sq},{Sk}]")
+        if drop_mask.dtype not in (torch.uint8, q.dtype) or not drop_mask.is_contiguous() or drop_mask.shape != (B, N, Sq, Sk):
+            raise TypeError(f"drop_mask must be contiguous [{B},{N},{Sq},{Sk}], uint8 or {q.dtype}")
         p.drop_mask = drop_mask.data_ptr()
+        p.drop_mask_kind = DROP_U8 if drop_mask.dtype == torch.uint8 else DROP_F16
         keep.append(drop_mask)
     if drop_seed is not None:
         if drop_mask is not None:
@@ -229,7 +234,10 @@ def fa_bwd(p, q, k, v, o, do, lse):
     if not q.is_cuda:
         raise RuntimeError("acct_fa_bwd needs device tensors (there is no CPU path)")
     if do.stride() != o.stride():
-        do = do.contiguous() if o.is_contiguous() else do.clone(memory_format=torch.preserve_format).as_strided(o.size(), o.stride())
+        # the kernels read dO with O's strides: copy the values into a buffer laid out like O
+        tmp = torch.empty_strided(o.size(), o.stride(), dtype=o.dtype, device=o.device)
+        tmp.copy_(do)
+        do = tmp
     p.o_stride = _bhs_strides(o)
     dq = torch.empty_strided(q.size(), q.stride(), dtype=q.dtype, device=q.device)
     dk = torch.empty_strided(k.size(), k.stride(), dtype=k.dtype, device=k.device)

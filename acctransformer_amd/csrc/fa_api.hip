@@ -49,6 +49,10 @@ size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 bool strides_zero(const int64_t s[3]) { return s[0] == 0 && s[1] == 0 && s[2] == 0; }
 
+bool mask_is_dense(const acct_fa_params* p) { return p->mask_kind == ACCT_MASK_DENSE_U8 || p->mask_kind == ACCT_MASK_DENSE_F16; }
+bool mask_is_tile(const acct_fa_params* p) { return p->mask_kind == ACCT_MASK_TILE_U8 || p->mask_kind == ACCT_MASK_TILE_F16; }
+int mask_elem_size(const acct_fa_params* p) { return (p->mask_kind == ACCT_MASK_DENSE_F16 || p->mask_kind == ACCT_MASK_TILE_F16) ? 2 : 1; }
+
 // counter-based dropout is on: the keep mask comes from (drop_seed, drop_offset), not from a tensor
 bool philox_on(const acct_fa_params* p) { return p->drop_philox != 0 && !p->drop_mask && p->keep_prob < 1.f; }
 bool dropout_on(const acct_fa_params* p) { return p->drop_mask != nullptr || philox_on(p); }
@@ -76,13 +80,16 @@ int validate(const acct_fa_params* p, bool backward) {
   if (p->row_block_prefix < 0 || p->row_block_prefix % 128 != 0) return fail(ACCT_E_PARAM, "row_block_prefix must be 0 or a positive multiple of 128, got %d", p->row_block_prefix);
   switch (p->mask_kind) {
     case ACCT_MASK_NONE: case ACCT_MASK_CAUSAL: break;
-    case ACCT_MASK_DENSE_U8: case ACCT_MASK_TILE_U8:
+    case ACCT_MASK_DENSE_U8: case ACCT_MASK_TILE_U8: case ACCT_MASK_DENSE_F16: case ACCT_MASK_TILE_F16:
       if (!p->attn_mask) return fail(ACCT_E_NULLPTR, "attn_mask is NULL but mask_kind=%d needs a tensor", p->mask_kind);
       break;
     default: return fail(ACCT_E_PARAM, "unknown mask_kind %d", p->mask_kind);
   }
-  if (p->mask_stride_b < 0 || (p->mask_kind == ACCT_MASK_DENSE_U8 && p->mask_stride_b != 0 && p->mask_stride_b < (int64_t)p->Sq * p->Sk))
+  if (p->mask_stride_b < 0 || (mask_is_dense(p) && p->mask_stride_b != 0 && p->mask_stride_b < (int64_t)p->Sq * p->Sk))
     return fail(ACCT_E_SHAPE, "mask_stride_b must be 0 (broadcast) or >= Sq*Sk");
+  if (mask_elem_size(p) == 2 && ((uintptr_t)p->attn_mask & 1)) return fail(ACCT_E_SHAPE, "a 2-byte attn_mask must be 2-byte aligned");
+  if (p->drop_mask_kind != ACCT_DROP_U8 && p->drop_mask_kind != ACCT_DROP_F16) return fail(ACCT_E_PARAM, "unknown drop_mask_kind %d", p->drop_mask_kind);
+  if (p->drop_mask && p->drop_mask_kind == ACCT_DROP_F16 && ((uintptr_t)p->drop_mask & 1)) return fail(ACCT_E_SHAPE, "a 2-byte drop_mask must be 2-byte aligned");
   if (!p->q || !p->k || !p->v) return fail(ACCT_E_NULLPTR, "q, k and v must be non-NULL");
   const int64_t* st[4] = {p->q_stride, p->k_stride, p->v_stride, p->o_stride};
   const void* ptrs[3] = {p->q, p->k, p->v};
@@ -109,8 +116,10 @@ acct::FaArgs make_args(const acct_fa_params* p) {
   acct::FaArgs a;
   memset(&a, 0, sizeof(a));
   a.q = p->q; a.k = p->k; a.v = p->v;
-  a.mask = (p->mask_kind == ACCT_MASK_DENSE_U8 || p->mask_kind == ACCT_MASK_TILE_U8) ? p->attn_mask : nullptr;
-  a.drop = p->keep_prob < 1.f || p->drop_mask ? p->drop_mask : nullptr;
+  a.mask = (mask_is_dense(p) || mask_is_tile(p)) ? (const uint8_t*)p->attn_mask : nullptr;
+  a.mask_es = mask_elem_size(p);
+  a.drop = p->keep_prob < 1.f || p->drop_mask ? (const uint8_t*)p->drop_mask : nullptr;
+  a.drop_es = p->drop_mask_kind == ACCT_DROP_F16 ? 2 : 1;
   a.alibi = p->alibi;
   a.B = p->B; a.N = p->N; a.Sq = p->Sq; a.Sk = p->Sk;
   a.Tr = (p->Sq + 127) / 128; a.Tc = (p->Sk + 127) / 128;
@@ -118,7 +127,7 @@ acct::FaArgs make_args(const acct_fa_params* p) {
   fill_strides(p->k_stride, p->N, p->Sk, p->D, &a.k_sb, &a.k_sh, &a.k_ss);
   fill_strides(p->v_stride, p->N, p->Sk, p->D, &a.v_sb, &a.v_sh, &a.v_ss);
   fill_strides(p->o_stride, p->N, p->Sq, p->D, &a.o_sb, &a.o_sh, &a.o_ss);
-  a.mask_sb = p->mask_kind == ACCT_MASK_DENSE_U8 ? p->mask_stride_b : 0;
+  a.mask_sb = mask_is_dense(p) ? p->mask_stride_b : 0;
   a.al_sb = p->alibi_stride_b; a.al_sh = p->alibi_stride_h; a.al_sq = p->alibi_stride_q;
   a.scale = p->scale;
   a.scale_log2e = p->scale * acct::kLog2e;
@@ -131,16 +140,26 @@ acct::FaArgs make_args(const acct_fa_params* p) {
     a.inv_keep = 256.0f / (float)a.philox_thr;          // the reciprocal of the keep probability actually used
   }
   a.inv_scale = 1.0f / p->scale;
+  {
+    // 2^p_shift grows with the key count (average probability 1 / Sk) and stops at 2^8, which leaves
+    // |dP - D| < 255 of headroom in fp16 for a row whose probability mass sits on one key
+    int lg = 0;
+    while ((2 << lg) <= p->Sk) lg++;
+    const int sh = lg - 9 < 0 ? 0 : (lg - 9 > 8 ? 8 : lg - 9);
+    a.p_shift = (float)sh;
+    a.p_unshift = 1.0f / (float)(1 << sh);
+  }
   a.mask_add_raw = acct::kMaskFill / p->scale;
   a.prev_blk = p->prev_block_num > ACCT_BLOCK_UNBOUNDED ? ACCT_BLOCK_UNBOUNDED : p->prev_block_num;
   a.next_blk = p->next_block_num > ACCT_BLOCK_UNBOUNDED ? ACCT_BLOCK_UNBOUNDED : p->next_block_num;
-  a.mask_kind = p->mask_kind;
+  // the kernels know one dense and one tile kind; the element size travels beside it
+  a.mask_kind = mask_is_dense(p) ? (int)acct::kMaskDense : (mask_is_tile(p) ? (int)acct::kMaskTile : p->mask_kind);
   a.row_prefix = p->row_block_prefix;
   return a;
 }
 
 size_t flag_bytes(const acct_fa_params* p) {
-  if (p->mask_kind != ACCT_MASK_DENSE_U8) return 0;
+  if (!mask_is_dense(p)) return 0;
   const size_t MB = p->mask_stride_b ? p->B : 1;
   return align_up(MB * (size_t)((p->Sq + 127) / 128) * (size_t)((p->Sk + 127) / 128), 256);
 }
@@ -152,8 +171,8 @@ hipError_t prepare_mask(acct::FaArgs& a, const acct_fa_params* p, uint8_t* flags
 
 // per-key-column bitmaps of the mixed blocks of a dense mask (backward only): 16 bytes per (q block, key)
 size_t colbit_bytes(const acct_fa_params* p) {
-  if (p->mask_kind == ACCT_MASK_TILE_U8) return 128 * 16;
-  if (p->mask_kind != ACCT_MASK_DENSE_U8) return 0;
+  if (mask_is_tile(p)) return 128 * 16;
+  if (!mask_is_dense(p)) return 0;
   const size_t MB = p->mask_stride_b ? p->B : 1;
   return align_up(MB * (size_t)((p->Sq + 127) / 128) * (size_t)p->Sk * 16, 256);
 }
@@ -167,11 +186,6 @@ size_t droprow_bytes(const acct_fa_params* p) {
 size_t dropcol_bytes(const acct_fa_params* p) {
   if (!dropout_on(p)) return 0;
   return align_up((size_t)p->B * p->N * (size_t)((p->Sq + 127) / 128) * (size_t)p->Sk * 16, 256);
-}
-
-int env_int(const char* name, int dflt) {
-  const char* s = getenv(name);
-  return s && *s ? atoi(s) : dflt;
 }
 
 }  // namespace
@@ -204,18 +218,19 @@ int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, s
   int rc = validate(p, false);
   if (rc) return rc;
   if (!O || !LSE) return fail(ACCT_E_NULLPTR, "O and LSE must be non-NULL");
-  if ((uintptr_t)O & 7) return fail(ACCT_E_SHAPE, "O must be 8-byte aligned");
+  if ((uintptr_t)O & 15) return fail(ACCT_E_SHAPE, "O must be 16-byte aligned");
   if (p->keep_prob < 1.f && !dropout_on(p)) return fail(ACCT_E_NULLPTR, "keep_prob < 1 needs a drop_mask or drop_philox");
   const size_t need = acct_fa_fwd_workspace_bytes(p);
   if (need && (!workspace || workspace_bytes < need))
     return fail(ACCT_E_WORKSPACE, "forward workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
+  if (need && ((uintptr_t)workspace & 255)) return fail(ACCT_E_WORKSPACE, "workspace must be 256-byte aligned");
   int n_cu = 0;
   rc = check_device(&n_cu);
   if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
   acct::FaArgs a = make_args(p);
   a.o = O; a.lse = LSE;
-  if (p->mask_kind == ACCT_MASK_DENSE_U8) {
+  if (mask_is_dense(p)) {
     hipError_t e = prepare_mask(a, p, (uint8_t*)workspace, st);
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
   }
@@ -233,7 +248,6 @@ int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, s
   // 8 waves x 32 query rows (two waves per SIMD overlap MFMA and softmax work) once that still
   // fills the chip, else 4 waves x 32 rows for more workgroups
   int qg = ((long long)p->B * p->N * ((p->Sq + 255) / 256) >= n_cu) ? 3 : 1;
-  qg = env_int("ACCT_FA_FWD_VARIANT", qg);
   hipError_t e = acct::launch_fwd(a, p->dtype, p->D, qg, st);
   if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "forward kernel: %s", hipGetErrorString(e));
   return ACCT_OK;
@@ -264,13 +278,13 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
   const size_t stat_bytes = align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256);
   a.delta = (float*)workspace;
   a.nlse = (float*)((char*)workspace + stat_bytes);
-  if (p->mask_kind == ACCT_MASK_DENSE_U8) {
+  if (mask_is_dense(p)) {
     uint8_t* flags = (uint8_t*)workspace + 2 * stat_bytes;
     // (the dkdv-only call re-derives the flags as well: the mask may have been edited since)
     hipError_t e = prepare_mask(a, p, flags, st);
     if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
   }
-  if (want_dkdv && (p->mask_kind == ACCT_MASK_DENSE_U8 || p->mask_kind == ACCT_MASK_TILE_U8)) {
+  if (want_dkdv && (mask_is_dense(p) || mask_is_tile(p))) {
     uint8_t* flags = (uint8_t*)workspace + 2 * stat_bytes;          // (no flags for the tile kind: flag_bytes = 0)
     uint32_t* cbits = (uint32_t*)(flags + flag_bytes(p));
     a.colbits = cbits;

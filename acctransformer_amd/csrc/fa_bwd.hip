@@ -19,18 +19,6 @@
 #include "fa_launch.hpp"
 
 namespace acct {
-
-ACCT_DEV void load_f32x4(const float* base, int idx, int limit, bool vec_ok, float fill, float out[4]) {
-  if (vec_ok && idx + 4 <= limit) {
-    const f32x4 t = *reinterpret_cast<const f32x4*>(base + idx);
-#pragma unroll
-    for (int e = 0; e < 4; e++) out[e] = t[e];
-  } else {
-#pragma unroll
-    for (int e = 0; e < 4; e++) out[e] = (idx + e < limit) ? base[idx + e] : fill;
-  }
-}
-
 template <typename T>
 ACCT_DEV typename Elem<T>::V8 pack8(const float* x) {
   using E = Elem<T>;
@@ -49,6 +37,8 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   using C = SwzCfg<D>;
   constexpr int BM = 32 * QG * NW;
   constexpr int TILEB = 64 * C::PITCH;
+  constexpr int FRING = 4, TRING = 3;                     // fragment reads in flight ahead of their MFMA (row-major / transposed)
+  constexpr bool RINGS = !(BIAS || DROP);                 // (the side-input variants have no registers for the rings)   // fragment reads in flight ahead of their MFMA (row-major / transposed)
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 buffers][K tile | V tile]; reused by the epilogue
 
@@ -109,10 +99,11 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
     dl[gq] = pair_sum(part);
     lq[gq] = INFINITY;                                   // rows past Sq: P = exp2(x - inf) = 0
     if (row < a.Sq) {
-      lq[gq] = a.lse[(int64_t)bh * a.Sq + row] * kLog2e;
+      // (minus p_shift: the recomputed probabilities carry a factor 2^p_shift, see FaArgs)
+      lq[gq] = a.lse[(int64_t)bh * a.Sq + row] * kLog2e - a.p_shift;
       if (g == 0) {
         a.delta[(int64_t)bh * a.Sq + row] = dl[gq];
-        a.nlse[(int64_t)bh * a.Sq + row] = -lq[gq];        // -LSE*log2(e): the exp2 offset the dK/dV kernel adds
+        a.nlse[(int64_t)bh * a.Sq + row] = -lq[gq];        // p_shift - LSE*log2(e): the exp2 offset the dK/dV kernel adds
       }
     }
   }
@@ -136,10 +127,10 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
       for (int r = 0; r < 16; r++) acc[gq][db][r] = 0.f;
 
   const int mb = a.mask_sb ? b : 0;
-  const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
+  const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb * a.mask_es : 0) : nullptr;
   const T* alibip = BIAS ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
-  const bool mask_vec = a.mask_kind == kMaskDense ? (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0
-                                                  : ((uintptr_t)a.mask & 3) == 0;
+  const bool mask_vec = a.mask_kind == kMaskDense ? ((((uintptr_t)a.mask / a.mask_es) | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0
+                                                  : ((uintptr_t)a.mask & (4 * a.mask_es - 1)) == 0;
   const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
   TileDma<T, D, 64, NW> kdma, vdma;
@@ -223,7 +214,28 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 #pragma unroll
             for (int r = 0; r < 16; r++) dp[gq][r] = 0.f;
           }
-          {
+          if constexpr (RINGS) {
+            // K and V fragments of the chunk travel through a ring of FRING register sets (FRING reads in
+            // flight ahead of the MFMA that consumes the oldest); S and dP MFMAs alternate.  The scheduling
+            // barriers keep the compiler from folding the ring back into read-wait-MFMA.
+            constexpr int NF = 2 * C::KS;
+            auto faddr = [&](int i) { return ((i & 1) ? vbuf : kbuf) + koff[i >> 1] + c * 32 * C::PITCH; };
+            V8 ring[FRING];
+#pragma unroll
+            for (int i = 0; i < FRING; i++) ring[i] = lds_read_frag<T>(faddr(i));
+#pragma unroll
+            for (int i = 0; i < NF; i++) {
+              const int t = i >> 1;
+              __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+              for (int gq = 0; gq < QG; gq++) {
+                if (i & 1) dp[gq] = E::mfma(ring[i % FRING], dof[gq][t], dp[gq]);
+                else s[gq] = E::mfma(ring[i % FRING], qf[gq][t], s[gq]);
+              }
+              if (i + FRING < NF) ring[i % FRING] = lds_read_frag<T>(faddr(i + FRING));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          } else {
             V8 kf[C::KS], vf[C::KS];
 #pragma unroll
             for (int t = 0; t < C::KS; t++) kf[t] = lds_read_frag<T>(kbuf + koff[t] + c * 32 * C::PITCH);
@@ -287,8 +299,8 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
                 for (int r4 = 0; r4 < 4; r4++) {
                   const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
                   uint32_t mbits;
-                  if (a.mask_kind == kMaskDense) mbits = load_u8x4(maskp + (int64_t)qrow_c * a.Sk, kv, a.Sk, mask_vec);
-                  else mbits = load_u8x4(maskp + (qrow_c & 127) * 128, kv & 127, 128, mask_vec);
+                  if (a.mask_kind == kMaskDense) mbits = load_mask4(maskp + (int64_t)qrow_c * a.Sk * a.mask_es, kv, a.Sk, mask_vec, a.mask_es);
+                  else mbits = load_mask4(maskp + (qrow_c & 127) * 128 * a.mask_es, kv & 127, 128, mask_vec, a.mask_es);
 #pragma unroll
                   for (int e = 0; e < 4; e++)
                     if ((mbits >> (8 * e)) & 0xffu) x[4 * r4 + e] += kMaskFill * kLog2e;
@@ -321,18 +333,39 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
             dsf[gq][c][1] = pack8<T>(ds + 8);
           }
         }
-        // ---- dQ^T += K^T dS^T ----
+        // ---- dQ^T += K^T dS^T : transposed K fragments through a ring of TRING register sets ----
+        if constexpr (RINGS) {
+          constexpr int NT = 4 * C::DB;
+          auto tread = [&](int i) {
+            const int db = i % C::DB, ch = i / C::DB;           // ch = 2 c + hh: rows 16 ch .. of the tile
+            const ACCT_LDS char* kaddr = kbuf + toff[db] + 16 * ch * C::PITCH;
+            return join_tr<T>(lds_read_tr(kaddr), lds_read_tr(kaddr + C::tr_hi(db)));
+          };
+          V8 ring[TRING];
 #pragma unroll
-        for (int c = 0; c < 2; c++)
+          for (int i = 0; i < TRING; i++) ring[i] = tread(i);
 #pragma unroll
-          for (int hh = 0; hh < 2; hh++)
+          for (int i = 0; i < NT; i++) {
+            const int db = i % C::DB, ch = i / C::DB;
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int db = 0; db < C::DB; db++) {
-              const ACCT_LDS char* kaddr = kbuf + toff[db] + (32 * c + 16 * hh) * C::PITCH;
-              const V8 ktf = join_tr<T>(lds_read_tr(kaddr), lds_read_tr(kaddr + C::tr_hi(db)));
+            for (int gq = 0; gq < QG; gq++) acc[gq][db] = E::mfma(ring[i % TRING], dsf[gq][ch >> 1][ch & 1], acc[gq][db]);
+            if (i + TRING < NT) ring[i % TRING] = tread(i + TRING);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        } else {
 #pragma unroll
-              for (int gq = 0; gq < QG; gq++) acc[gq][db] = E::mfma(ktf, dsf[gq][c][hh], acc[gq][db]);
-            }
+          for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+              for (int db = 0; db < C::DB; db++) {
+                const ACCT_LDS char* kaddr = kbuf + toff[db] + (32 * c + 16 * hh) * C::PITCH;
+                const V8 ktf = join_tr<T>(lds_read_tr(kaddr), lds_read_tr(kaddr + C::tr_hi(db)));
+#pragma unroll
+                for (int gq = 0; gq < QG; gq++) acc[gq][db] = E::mfma(ktf, dsf[gq][c][hh], acc[gq][db]);
+              }
+        }
       } else if (BIAS && bias_staged && j < j_hi && wq0 < a.Sq) {
         stage_bias(j + 1);                                  // nothing to read in this step: the region is free
       }
@@ -342,6 +375,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   }
 
   // ---- epilogue: dQ = scale * dQ^T, transposed through the wave's own LDS region ----
+  const float dq_scale = a.scale * a.p_unshift;
   T* dqp = (T*)a.dq + b * a.q_sb + h * a.q_sh;
   constexpr int OPITCH = C::DB * 64 + 16;
   ACCT_LDS char* obuf = smem + wave * (32 * OPITCH);
@@ -351,8 +385,8 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
     for (int db = 0; db < C::DB; db++)
 #pragma unroll
       for (int r4 = 0; r4 < 4; r4++) {
-        typename E::V2 t0 = E::cvt2(acc[gq][db][4 * r4 + 0] * a.scale, acc[gq][db][4 * r4 + 1] * a.scale);
-        typename E::V2 t1 = E::cvt2(acc[gq][db][4 * r4 + 2] * a.scale, acc[gq][db][4 * r4 + 3] * a.scale);
+        typename E::V2 t0 = E::cvt2(acc[gq][db][4 * r4 + 0] * dq_scale, acc[gq][db][4 * r4 + 1] * dq_scale);
+        typename E::V2 t1 = E::cvt2(acc[gq][db][4 * r4 + 2] * dq_scale, acc[gq][db][4 * r4 + 3] * dq_scale);
         typename E::V4 ov = {t0[0], t0[1], t1[0], t1[1]};
         *reinterpret_cast<ACCT_LDS typename E::V4*>(obuf + l32 * OPITCH + (32 * db + 8 * r4 + 4 * g) * 2) = ov;
       }
@@ -380,15 +414,11 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 // (two waves fit on each SIMD and overlap each other's MFMA and exp/convert
 // phases) while every Q / dO fragment read from LDS still feeds two MFMAs.
 // ============================================================================
-#ifndef ACCT_PARK
-#define ACCT_PARK 6
-#endif
-#ifndef ACCT_PARK_HOT
-#define ACCT_PARK_HOT 4      // the variant without side inputs has registers for two more fragments
-#endif
+constexpr int kPark = 6;        // stationary fragments parked in LDS per wave (D = 128)
+constexpr int kParkHot = 4;     // the variant without side inputs has registers for two more fragments
 // stationary fragments parked in LDS per wave: the bias variants give one up for the bias tiles' LDS
 template <int D, bool BIAS, bool MASKT>
-constexpr int dkdv_park() { return D >= 128 ? (BIAS ? ACCT_PARK - 1 : (MASKT ? ACCT_PARK : ACCT_PARK_HOT)) : 0; }
+constexpr int dkdv_park() { return D >= 128 ? (BIAS ? kPark - 1 : (MASKT ? kPark : kParkHot)) : 0; }
 
 // MASKT = false compiles the mask-tensor handling out (no mask, or the causal mask by index compare):
 // the hot variant must not carry that code's register pressure.
@@ -476,14 +506,9 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   // per-lane LDS offsets (tile-invariant)
 #define FOFF(t) (foff4[(t) & 3] ^ (((t) >> 2) * 128))
 #define TOFF(db) (toff2[(db) & 1] + ((db) >> 1) * 128)
-#ifdef ACCT_NO_EDGE
-#define EDGE_PATH false
-#else
-#define EDGE_PATH edge
-#endif
 
   const int mb = a.mask_sb ? b : 0;
-  const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
+  const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb * a.mask_es : 0) : nullptr;
   const T* alibip = BIAS ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
 
   // stage q tile i into buffer `sb`: Q and dO by 16-byte DMA (2 instructions per wave each),
@@ -568,13 +593,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     const uint8_t* flcol = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + (int64_t)mb * a.Tr * a.Tc + wkb : nullptr;
     BlkClassWindow flwin;
     flwin.init(flcol, a.Tc, c_lo >> 2, c_hi >> 2, lane);
-#ifdef ACCT_TRACE
-#define TR(k) if (blockIdx.x == ACCT_TRACE && lane == 0 && n - c_lo < 96) ((unsigned long long*)((char*)a.delta + 2 * (size_t)a.B * a.N * a.Sq * 4))[((wave * 96) + (n - c_lo)) * 8 + (k)] = __builtin_amdgcn_s_memtime()
-#else
-#define TR(k)
-#endif
     for (int n = c_lo; n <= c_hi + 1; n++) {
-      TR(0);
       if ((n & 1) && (n >> 1) < i_hi) stage((n >> 1) + 1, smem + ((((n >> 1) + 1 - i_lo) & 1) * STAGEB));
       const int cidx = __builtin_amdgcn_readfirstlane(krole ? n - 1 : n);   // the chunk this wave works on in this step (wave-uniform: scalar)
       if (cidx >= c_lo && cidx <= c_hi) {
@@ -630,26 +649,28 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
               for (int r = 0; r < 16; r++) t0[gk][r] = 0.f;
           }
           {
-            // software pipeline: the fragments of k-step t+1 are requested before the MFMAs of k-step t
+            // software pipeline: the A fragments travel through a ring of ARING register sets (ARING reads in
+            // flight ahead of the MFMAs that consume the oldest), the parked B fragment is requested one
+            // k-step ahead
+            constexpr int ARING = 2;
             const ACCT_LDS char* abuf = (krole ? dobuf : qbuf) + c * 32 * C::PITCH;
-            V8 af = lds_read_frag<T>(abuf + FOFF(0));
+            V8 ar[ARING];
+#pragma unroll
+            for (int t = 0; t < ARING; t++) ar[t] = lds_read_frag<T>(abuf + FOFF(t));
             V8 b1 = (0 >= C::KS - PARK) ? *reinterpret_cast<const ACCT_LDS V8*>(park) : bf[1][0];
 #pragma unroll
             for (int t = 0; t < C::KS; t++) {
-              V8 afn = af, b1n = b1;
-              if (t + 1 < C::KS) {
-                afn = lds_read_frag<T>(abuf + FOFF(t + 1));
+              V8 b1n = b1;
+              if (t + 1 < C::KS)
                 b1n = (t + 1 >= C::KS - PARK) ? *reinterpret_cast<const ACCT_LDS V8*>(park + (t + 1 - (C::KS - PARK)) * 1024) : bf[1][t + 1];
-              }
               __builtin_amdgcn_sched_barrier(0);
-              t0[0] = E::mfma(af, bf[0][t], t0[0]);                                         // S[q, key] or dP[q, key]
-              t0[1] = E::mfma(af, b1, t0[1]);
+              t0[0] = E::mfma(ar[t % ARING], bf[0][t], t0[0]);                              // S[q, key] or dP[q, key]
+              t0[1] = E::mfma(ar[t % ARING], b1, t0[1]);
               __builtin_amdgcn_sched_barrier(0);
-              af = afn;
+              if (t + ARING < C::KS) ar[t % ARING] = lds_read_frag<T>(abuf + FOFF(t + ARING));
               b1 = b1n;
             }
           }
-          TR(1);
           if (BIAS && bias_staged) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // bias tile consumed: stage the next chunk's
             if (n < c_hi) stage_bias(n + 1);
@@ -662,7 +683,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
           }
           V8 bfr[2][2];                               // B fragments of the second product: P (V role) or dS (K role)
           if (!krole) {
-            if (EDGE_PATH) {
+            if (edge) {
               // Side inputs and range limits are folded into the raw scores in place, in three short
               // passes that each keep few values live: + bias/scale (unstaged bias only); - 10000/scale where the mask bit of
               // (row, key) is set; -inf where the key comes after the query (causal) or where the key
@@ -760,35 +781,42 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
               }
             }
           }
-          TR(2);
           // dV^T += dO^T P (V role) ; dK^T += Q^T dS (K role): contract over the 32 query rows of the chunk
           const ACCT_LDS char* tb = (krole ? qbuf : dobuf) + c * 32 * C::PITCH;
-#pragma unroll
-          for (int hh = 0; hh < 2; hh++)
-#pragma unroll
-            for (int db = 0; db < C::DB; db++) {
+          {
+            // transposed fragments through a ring of BRING register sets, as above
+            constexpr int BRING = 2, NT = 2 * C::DB;
+            auto tread = [&](int i) {
+              const int db = i % C::DB, hh = i / C::DB;
               const ACCT_LDS char* ta = tb + TOFF(db) + 16 * hh * C::PITCH;
-              const V8 af = join_tr<T>(lds_read_tr(ta), lds_read_tr(ta + C::tr_hi(db)));
+              return join_tr<T>(lds_read_tr(ta), lds_read_tr(ta + C::tr_hi(db)));
+            };
+            V8 tr[BRING];
 #pragma unroll
-              for (int gk = 0; gk < 2; gk++) acc[gk][db] = E::mfma(af, bfr[gk][hh], acc[gk][db]);
+            for (int i = 0; i < BRING; i++) tr[i] = tread(i);
+#pragma unroll
+            for (int i = 0; i < NT; i++) {
+              const int db = i % C::DB, hh = i / C::DB;
+              __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+              for (int gk = 0; gk < 2; gk++) acc[gk][db] = E::mfma(tr[i % BRING], bfr[gk][hh], acc[gk][db]);
+              __builtin_amdgcn_sched_barrier(0);
+              if (i + BRING < NT) tr[i % BRING] = tread(i + BRING);
             }
+          }
         } else if (BIAS && bias_staged && n < c_hi) {
           stage_bias(n + 1);                            // nothing to read in this step: the region is free
         }
       }
-      TR(3);
       dma_wait();                                     // a tile requested at the top of this step has landed
-      TR(4);
       __syncthreads();
-      TR(5);
     }
-#undef TR
   }
 
   // ---- epilogue: dV (V role) / scale * dK (K role), transposed through the wave's own LDS region ----
   T* outp = krole ? (T*)a.dk + b * a.k_sb + h * a.k_sh : (T*)a.dv + b * a.v_sb + h * a.v_sh;
   const int64_t oss = krole ? a.k_ss : a.v_ss;
-  const float oscale = krole ? a.scale : (DROP ? a.inv_keep : 1.0f);
+  const float oscale = (krole ? a.scale : (DROP ? a.inv_keep : 1.0f)) * a.p_unshift;
   constexpr int OPITCH = C::DB * 64 + 16;
   ACCT_LDS char* obuf = smem + wave * (32 * OPITCH);
 #pragma unroll
@@ -818,7 +846,6 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 
 #undef FOFF
 #undef TOFF
-#undef EDGE_PATH
 
 // ---- launchers ----------------------------------------------------------------
 template <typename T, int D, bool BIAS, bool DROP>
@@ -833,7 +860,7 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
     a.n_tiles = (a.Sq + BM - 1) / BM;
     const bool mask_q = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;
     auto kern = mask_q ? fa_bwd_dq_kernel<T, D, QG, NW, BIAS, DROP, true> : fa_bwd_dq_kernel<T, D, QG, NW, BIAS, DROP, BIAS || DROP>;
-    e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    e = allow_dynamic_lds((const void*)kern, smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)((long long)a.n_tiles * a.B * a.N)), dim3(64 * NW), smem, st, a);
     e = hipGetLastError();
@@ -849,7 +876,7 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
     a.n_tiles = (a.Sk + 255) / 256;
     const bool mask_t = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;
     auto kern = mask_t ? fa_bwd_dkdv_kernel<T, D, BIAS, DROP, true> : fa_bwd_dkdv_kernel<T, D, BIAS, DROP, BIAS || DROP>;
-    e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem2);
+    e = allow_dynamic_lds((const void*)kern, smem2);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)((long long)a.n_tiles * a.B * a.N)), dim3(512), smem2, st, a);
     e = hipGetLastError();

@@ -26,7 +26,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #define ACCT_DEV __device__ __forceinline__
 
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kMaskFill = -10000.0f;   // additive mask value of the reference (constants.py:24)
 
 // ---- element-type traits ---------------------------------------------------
@@ -106,7 +105,7 @@ struct FaArgs {
   void* o; float* lse;                 // fwd outputs / bwd inputs
   const void* dout; void* dq; void* dk; void* dv;                // bwd only
   float* delta; float* nlse;           // bwd workspace: D = rowsum(dO*O) and -LSE*log2(e), [B,N,Sq] each
-  const uint8_t* mask; const uint8_t* drop; const void* alibi;
+  const uint8_t* mask; const uint8_t* drop; const void* alibi;   // mask / drop: elements of mask_es / drop_es bytes
   const uint8_t* blkflags;             // [MB, Tr, Tc] block classes of a dense mask
   const uint32_t* droprow;             // [B*N*Sq, droprow_w] keep bits of the dropout mask by query row: bit k of word w = drop[row][32w+k] != 0
   const uint32_t* dropcol;             // [B*N, Tr, Sk, 4] the same by key column: bit r of the 128-bit entry = drop[128*qb + r][key] != 0
@@ -122,8 +121,13 @@ struct FaArgs {
   int64_t al_sb, al_sh, al_sq;
   float scale, scale_log2e, inv_keep, inv_scale;
   float mask_add_raw;                  // -10000 / scale: the mask in raw q.k units
+  // The backward recomputes P = exp(S - LSE), normalised: with many keys its entries, and dS = P (dP - D), fall
+  // into the subnormal range of fp16 before they feed the MFMAs.  The kernels therefore work with 2^p_shift P
+  // (a shift of the exp2 argument: no instruction) and multiply dQ, dK, dV by p_unshift = 2^-p_shift at the end.
+  float p_shift, p_unshift;
   int prev_blk, next_blk;
   int mask_kind;
+  int mask_es, drop_es;                // bytes per element of mask and drop: 1 (uint8) or 2 (the I/O dtype); nonzero = masked / kept
   int row_prefix;                      // >0: row i sees keys j < (i/row_prefix + 1)*row_prefix only (multiple of 128)
   int n_tiles;                         // tiles along the owner dimension
   int droprow_w;                       // 32-bit words per row of droprow: 2 * ceil(Sk / 64)
@@ -209,6 +213,29 @@ ACCT_DEV uint32_t load_u8x4(const uint8_t* row, int kv, int limit, bool vec_ok) 
   return r;
 }
 
+// mask / dropout element -> "is nonzero": a 2-byte element is a floating-point number, whose zero may carry a sign
+template <int ES> ACCT_DEV bool elem_nonzero(const uint8_t* p, int64_t idx) {
+  if (ES == 1) return p[idx] != 0;
+  return (reinterpret_cast<const uint16_t*>(p)[idx] & 0x7fffu) != 0;
+}
+// the same four consecutive elements for a mask of `es`-byte elements, as four "nonzero" bytes (row = first byte of the row)
+ACCT_DEV uint32_t load_mask4(const uint8_t* row, int kv, int limit, bool vec_ok, int es) {
+  if (es == 1) return load_u8x4(row, kv, limit, vec_ok);
+  const uint16_t* r16 = reinterpret_cast<const uint16_t*>(row);
+  uint32_t r = 0;
+  if (vec_ok && kv + 4 <= limit) {
+    const u32x2 t = *reinterpret_cast<const u32x2*>(r16 + kv);
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      if ((t[e >> 1] >> (16 * (e & 1))) & 0x7fffu) r |= 1u << (8 * e);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      if (kv + e < limit && (r16[kv + e] & 0x7fffu)) r |= 1u << (8 * e);
+  }
+  return r;
+}
+
 template <typename T>
 ACCT_DEV void load_bias4(const T* row, int kv, int limit, bool vec_ok, float out[4]) {
   if (vec_ok && kv + 4 <= limit) {
@@ -218,43 +245,6 @@ ACCT_DEV void load_bias4(const T* row, int kv, int limit, bool vec_ok, float out
   } else {
 #pragma unroll
     for (int e = 0; e < 4; e++) out[e] = (kv + e < limit) ? (float)row[kv + e] : 0.f;
-  }
-}
-
-// ---- 64-row tiles staged through LDS ---------------------------------------
-template <int D, int NT = 256> struct TileCfg {
-  static constexpr int KS = D / 16;             // 16-wide k-steps across the head dim
-  static constexpr int DB = (D + 31) / 32;      // 32-wide blocks across the head dim
-  static constexpr int DP = DB * 32;
-  static constexpr int CPR = D / 8;             // 16-byte chunks per row
-  static constexpr int ROWB = DP * 2 + 16;      // LDS row pitch (bytes): +16 keeps b128 reads conflict free
-  static constexpr int BN = 64;                 // rows per staged tile
-  static constexpr int TILEB = BN * ROWB;
-  static constexpr int NLD = (BN * CPR + NT - 1) / NT;   // 16-byte chunks per thread and tile
-};
-
-template <typename T, int D, int NT = 256>
-ACCT_DEV void tile_load(const T* base, int64_t row_stride, int row0, int nrows, u32x4 (&reg)[TileCfg<D, NT>::NLD]) {
-  using C = TileCfg<D, NT>;
-#pragma unroll
-  for (int i = 0; i < C::NLD; i++) {
-    const int idx = threadIdx.x + NT * i;
-    const int row = idx / C::CPR, ch = idx % C::CPR;
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (idx < C::BN * C::CPR && row0 + row < nrows)
-      v = *reinterpret_cast<const u32x4*>(base + (int64_t)(row0 + row) * row_stride + ch * 8);
-    reg[i] = v;
-  }
-}
-
-template <int D, int NT = 256>
-ACCT_DEV void tile_store(ACCT_LDS char* buf, const u32x4 (&reg)[TileCfg<D, NT>::NLD]) {
-  using C = TileCfg<D, NT>;
-#pragma unroll
-  for (int i = 0; i < C::NLD; i++) {
-    const int idx = threadIdx.x + NT * i;
-    const int row = idx / C::CPR, ch = idx % C::CPR;
-    if (idx < C::BN * C::CPR) *reinterpret_cast<ACCT_LDS u32x4*>(buf + row * C::ROWB + ch * 16) = reg[i];
   }
 }
 
@@ -294,14 +284,15 @@ template <int D> struct SwzCfg {
 // tile with NW waves.  Rows past nrows repeat the last valid row (finite data whose
 // contribution is zeroed by the caller's masking), slots past the valid chunks
 // repeat the last valid chunk.
+// `wv` < 0: the NW waves are the workgroup's first NW; else the calling wave's index among the NW.
 template <typename T, int D, int ROWS, int NW>
-ACCT_DEV void tile_dma(const T* base, int64_t row_stride, int row0, int nrows, ACCT_LDS char* buf) {
+ACCT_DEV void tile_dma(const T* base, int64_t row_stride, int row0, int nrows, ACCT_LDS char* buf, int wv = -1) {
   using C = SwzCfg<D>;
   constexpr int NI = ROWS / C::RPI;
   static_assert(NI % NW == 0, "tile rows must split evenly over the waves");
   int tid = threadIdx.x;
   asm volatile("" : "+v"(tid));                   // addresses are re-derived per call instead of living in registers
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63, wave = wv < 0 ? tid >> 6 : wv;
 #pragma unroll
   for (int i = 0; i < NI / NW; i++) {
     const int inst = wave * (NI / NW) + i;
@@ -327,13 +318,19 @@ struct TileDma {
   using C = SwzCfg<D>;
   static constexpr int NI = ROWS / C::RPI;
   static constexpr int NIW = NI / NW;              // instructions per wave and tile
-  uint32_t voff[NIW];
+  // The swizzle repeats every 16 rows, i.e. every PER instructions: instruction i of a wave differs from
+  // instruction i % PER by a whole number of 16-row groups, which goes into the scalar base address.
+  static constexpr int PER = 16 / C::RPI;
+  static constexpr int NV = NIW < PER ? NIW : PER;
+  static_assert(NIW <= PER || NIW % PER == 0, "a wave's share of a tile must be whole 16-row groups");
+  uint32_t voff[NV];
   uint32_t lds0;                                   // LDS byte offset of this wave's first 1 KB slab within a tile
-  ACCT_DEV void plan(int64_t row_stride) {
+  // `wv` < 0: the NW waves are the workgroup's first NW; else the calling wave's index among the NW
+  ACCT_DEV void plan(int64_t row_stride, int wv = -1) {
     static_assert(NI % NW == 0, "tile rows must split evenly over the waves");
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wv < 0 ? (int)(threadIdx.x >> 6) : wv;
 #pragma unroll
-    for (int i = 0; i < NIW; i++) {
+    for (int i = 0; i < NV; i++) {
       const int inst = wave * NIW + i;
       const int r = inst * C::RPI + lane / C::CH;
       const int lc = min((lane % C::CH) ^ C::swz(r), C::CPR - 1);
@@ -367,18 +364,21 @@ struct TileDma {
   }
   // rows [row0, row0 + ROWS) must exist
   ACCT_DEV void issue(const T* base, int64_t row_stride, int row0, ACCT_LDS char* buf) const {
-    const T* tile = base + (int64_t)row0 * row_stride;            // uniform: must live in scalar registers
-    {
-      const uint64_t t = (uint64_t)(uintptr_t)tile;               // (pinned there: under register pressure the
-      const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)t);          // compiler may hold it in VGPRs)
-      const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(t >> 32));
-      tile = (const T*)(uintptr_t)(((uint64_t)hi << 32) | lo);
-    }
     const uint32_t dst0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)buf) + lds0;
 #pragma unroll
-    for (int i = 0; i < NIW; i++)
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff[i]), "s"(tile), "s"(dst0 + i * 1024)
-                   : "memory");
+    for (int grp = 0; grp < (NIW + PER - 1) / PER; grp++) {
+      const T* tile = base + (int64_t)(row0 + 16 * grp) * row_stride;   // uniform: must live in scalar registers
+      {
+        const uint64_t t = (uint64_t)(uintptr_t)tile;               // (pinned there: under register pressure the
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)t);          // compiler may hold it in VGPRs)
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(t >> 32));
+        tile = (const T*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+      }
+#pragma unroll
+      for (int i = 0; i < NV; i++)
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff[i]), "s"(tile), "s"(dst0 + (grp * PER + i) * 1024)
+                     : "memory");
+    }
   }
 };
 

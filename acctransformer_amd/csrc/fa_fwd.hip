@@ -22,6 +22,7 @@ template <typename T, int D, int QG, int NW, bool BIAS, bool DROP, bool MASKT, i
 __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   static_assert(KT == 2 || (KT == 4 && !BIAS), "key tiles are 64 rows, or 128 rows in the variants without bias");
   constexpr int BN = 32 * KT;                       // key rows per tile
+  constexpr int FRING = 4, VRING = 3;   // fragment reads in flight ahead of their MFMA (K row-major / V transposed)
   constexpr int TPB = 128 / BN;                     // tiles per 128-column block
   using E = Elem<T>;
   using V8 = typename E::V8;
@@ -86,9 +87,13 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   }
 
   // ---- per-lane LDS offsets (tile-invariant) ----
-  int koff[C::KS];                                          // K fragment of k-step t: row l32, chunk 2t + g
+  // K fragment of k-step t: row l32, chunk 2t + g.  Chunk c + 8 of a row sits in slot (c ^ swz) ^ 8, so the
+  // offsets of the upper half of the head dim are one XOR away from the lower four (wide rows only).
+  constexpr int NKOFF = (C::CH >= 16 && C::KS > 4) ? 4 : C::KS;
+  int koff_[NKOFF];
 #pragma unroll
-  for (int t = 0; t < C::KS; t++) koff[t] = l32 * C::PITCH + swz_off(2 * t + g, C::swz(l32));
+  for (int t = 0; t < NKOFF; t++) koff_[t] = l32 * C::PITCH + swz_off(2 * t + g, C::swz(l32));
+  auto koff = [&](int t) { return t < NKOFF ? koff_[t] : (koff_[t & 3] ^ ((t >> 2) * 128)); };
   const int trow = 4 * g + ((lane & 15) >> 2);              // transposed reads: row within an 8-row group
   const int tchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
   int voff[C::DB];                                          // V^T fragment of d block db
@@ -114,10 +119,10 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   const float madd = BIAS ? kMaskFill : a.mask_add_raw;            // the additive -10000 in the units of s
   const float lazy_thr = 8.0f / cmul;                              // 8 octaves, in the units of s
   const int mb = a.mask_sb ? b : 0;
-  const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb : 0) : nullptr;
+  const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb * a.mask_es : 0) : nullptr;
   const T* alibip = BIAS ? (const T*)a.alibi + b * a.al_sb + h * a.al_sh : nullptr;
-  const bool mask_vec = a.mask_kind == kMaskDense ? (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0
-                                                  : ((uintptr_t)a.mask & 3) == 0;
+  const bool mask_vec = a.mask_kind == kMaskDense ? ((((uintptr_t)a.mask / a.mask_es) | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0
+                                                  : ((uintptr_t)a.mask & (4 * a.mask_es - 1)) == 0;
   const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
   TileDma<T, D, BN, NW> kdma, vdma;
@@ -134,6 +139,214 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   // keep bits of this wave's rows and one tile, staged with the tile's DMA (double buffered)
   using DropStage = DropRowStage<DROP, QG, KT>;
   ACCT_LDS char* drop_lds = smem + 4 * TILEB + (BIAS ? NW * QG * 4096 : 0) + wave * (2 * DropStage::BYTES);
+  // ---- the phases of a tile step: classification, S^T = K Q^T, online softmax, O^T += V^T P^T ----
+  const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
+  BlkClassWindow flwin;                                      // block classes of a dense mask: 64 blocks at a time in scalar registers
+  if (j_lo <= j_hi) flwin.init(flrow, 1, j_lo / TPB, j_hi / TPB, lane);
+  enum : uint32_t { kAct = 1u, kApply = 2u, kDiag = 4u };
+  // what this wave does with tile j (tiles must be asked for in ascending order)
+  auto classify = [&](int j) -> uint32_t {
+    const uint32_t fl_cur = flwin.get(j / TPB, lane);
+    const int kv0 = j * BN, kvb = j / TPB;
+    bool act = (kvb - a.next_blk <= wqb) && (wqb <= kvb + a.prev_blk) && (wq0 < a.Sq);
+    if (causal) act = act && (kv0 <= wq_end - 1);
+    act = act && (kv0 < wkv_limit);
+    bool apply_mask = false;
+    bool diag = causal;                                     // keys after the query are hidden, by index compare
+    if (MASKT && a.mask_kind == kMaskDense && act) {
+      act = fl_cur != kBlkSkip;
+      apply_mask = fl_cur == kBlkApply;
+      if (fl_cur == kBlkTriu) { diag = true; act = kv0 <= wq_end - 1; }
+    } else if (MASKT && a.mask_kind == kMaskTile) {
+      apply_mask = wqb == kvb;
+    }
+    return (act ? kAct : 0u) | (apply_mask ? kApply : 0u) | (diag ? kDiag : 0u);
+  };
+  // stage key rows [j BN, (j+1) BN) of K or V into an LDS tile
+  auto stage_tile = [&](const TileDma<T, D, BN, NW>& dma, const T* base, int64_t ss, int j, ACCT_LDS char* dst) {
+    if ((j + 1) * BN <= a.Sk) dma.issue(base, ss, j * BN, dst);
+    else tile_dma<T, D, BN, NW>(base, ss, j * BN, a.Sk, dst);   // ragged last tile: clamped rows
+  };
+  // S^T = K Q^T : s[gq][c] is the 32(kv) x 32(q) tile of kv chunk c
+  auto gemm_s = [&](const ACCT_LDS char* kbuf, f32x16 (&s)[QG][KT]) {
+#pragma unroll
+    for (int gq = 0; gq < QG; gq++)
+#pragma unroll
+      for (int c = 0; c < KT; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[gq][c][r] = 0.f;
+    // K fragments travel through a ring of FRING register sets: FRING reads are in flight ahead of the
+    // MFMA that consumes the oldest one, so that a wave covers the LDS latency (well over one MFMA) by
+    // itself.  The scheduling barriers keep the compiler from folding the ring back into read-wait-MFMA.
+    constexpr int NF = KT * C::KS;
+    constexpr int RING = FRING < NF ? FRING : NF;
+    V8 ring[RING];
+    auto kread = [&](int i) { return lds_read_frag<T>(kbuf + koff(i % C::KS) + (i / C::KS) * 32 * C::PITCH); };
+#pragma unroll
+    for (int i = 0; i < RING; i++) ring[i] = kread(i);
+#pragma unroll
+    for (int i = 0; i < NF; i++) {
+      const int c = i / C::KS, t = i % C::KS;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int gq = 0; gq < QG; gq++) s[gq][c] = E::mfma(ring[i % RING], qf[gq][t], s[gq][c]);
+      if (i + RING < NF)
+        ring[i % RING] = kread(i + RING);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // O^T += V^T P^T, the transposed V fragments through a ring as well
+  auto gemm_pv = [&](const ACCT_LDS char* vbuf, const V8 (&pf)[QG][KT][2]) {
+    constexpr int NT = 2 * KT * C::DB;
+    constexpr int RING = VRING < NT ? VRING : NT;
+    auto tread = [&](int i) {
+      const int db = i % C::DB, ch = i / C::DB;               // ch = 2 c + hh: rows 16 ch .. of the tile
+      const ACCT_LDS char* vaddr = vbuf + voff[db] + 16 * ch * C::PITCH;
+      return join_tr<T>(lds_read_tr(vaddr), lds_read_tr(vaddr + C::tr_hi(db)));
+    };
+    V8 ring[RING];
+#pragma unroll
+    for (int i = 0; i < RING; i++) ring[i] = tread(i);
+#pragma unroll
+    for (int i = 0; i < NT; i++) {
+      const int db = i % C::DB, ch = i / C::DB;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int gq = 0; gq < QG; gq++) o[gq][db] = E::mfma(ring[i % RING], pf[gq][ch >> 1][ch & 1], o[gq][db]);
+      if (i + RING < NT) ring[i % RING] = tread(i + RING);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // online softmax of the scores of tile j -> P^T fragments; `buf` = parity of the tile's staging buffers
+  auto softmax = [&](int j, int buf, uint32_t info, f32x16 (&s)[QG][KT], V8 (&pf)[QG][KT][2]) {
+    const int kv0 = j * BN;
+    const bool apply_mask = MASKT && (info & kApply), diag = info & kDiag;
+    // element (gq, c, r): q = wq0 + 32 gq + l32 ; kv = kv0 + 32 c + 8 (r/4) + 4 g + r%4
+    const bool edge = apply_mask || (diag && (kv0 + BN - 1 > wq0)) || (kv0 + BN > a.Sk);
+#pragma unroll
+    for (int gq = 0; gq < QG; gq++) {
+      const int qrow = wq0 + 32 * gq + l32;
+      const int qrow_c = min(qrow, a.Sq - 1);            // clamped for side-input addressing
+      if (BIAS) {
+        if (bias_staged) {
+          typename E::V4 bv[2][4];
+#pragma unroll
+          for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) bv[c][r4] = bias_tile_read<T>(bias_lds + gq * 4096, l32, 4 * c + r4, g);
+          if (gq == QG - 1) {
+            // the tile is in registers: its LDS region can take the next tile, which has the rest of
+            // this step to land (the end-of-step wait covers it)
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (j < j_hi) stage_bias(j + 1);
+          }
+#pragma unroll
+          for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++)
+#pragma unroll
+              for (int e = 0; e < 4; e++)
+                s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale, (float)bv[c][r4][e]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+              const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
+              float bias[4];
+              load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
+#pragma unroll
+              for (int e = 0; e < 4; e++)
+                s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale, bias[e]);
+            }
+        }
+      }
+      if (edge) {
+        if (apply_mask) {
+#pragma unroll
+          for (int c = 0; c < KT; c++)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+              const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
+              uint32_t mbits;
+              if (a.mask_kind == kMaskDense) mbits = load_mask4(maskp + (int64_t)qrow_c * a.Sk * a.mask_es, kv, a.Sk, mask_vec, a.mask_es);
+              else mbits = load_mask4(maskp + (qrow_c & 127) * 128 * a.mask_es, kv & 127, 128, mask_vec, a.mask_es);
+#pragma unroll
+              for (int e = 0; e < 4; e++)
+                if ((mbits >> (8 * e)) & 0xffu) s[gq][c][4 * r4 + e] += madd;
+            }
+        }
+        {
+          // Keys after the query (causal diagonal) and keys past Sk are removed outright: with the additive
+          // mask their probability underflows to exactly 0 as well (the diagonal key is always visible), so
+          // the result is the same bit for bit at a third of the vector instructions.
+          int vis = a.Sk - 1 - kv0 - 4 * g;                  // last visible key, relative to this lane's first
+          if (diag) vis = min(vis, qrow - kv0 - 4 * g);
+#pragma unroll
+          for (int c = 0; c < KT; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+              if (32 * c + 8 * (r >> 2) + (r & 3) > vis) s[gq][c][r] = -INFINITY;
+        }
+      }
+      // ---- online softmax for query row qrow ----
+      float mx = s[gq][0][0];
+#pragma unroll
+      for (int c = 0; c < KT; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[gq][c][r]);
+      mx = pair_max(mx);
+      // Lazy running max: it only moves when a score beats it by more than 2^8 in probability
+      // terms.  Until then P = exp2(s - m) may reach 256 instead of 1 (harmless in fp16/bf16 and in
+      // the fp32 sums; O = acc / l and LSE = m + ln l are unchanged), and the O rescale below is
+      // skipped for almost every tile after the first.
+      const bool grow = mx > m[gq] + lazy_thr;
+      const float m_new = grow ? mx : m[gq];
+      const float alpha = grow ? fast_exp2((m[gq] - m_new) * cmul) : 1.0f;
+      const float mc = m_new * cmul;
+      m[gq] = m_new;
+      float rs = 0.f;
+      float p[KT][16];
+#pragma unroll
+      for (int c = 0; c < KT; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          p[c][r] = fast_exp2(__builtin_fmaf(s[gq][c][r], cmul, -mc));
+          rs += p[c][r];
+        }
+      lsum[gq] = lsum[gq] * alpha + rs;                  // row sum BEFORE dropout
+      if (DROP) {
+        // keep bits of this row and tile: word c covers keys kv0 + 32c .. +31
+#pragma unroll
+        for (int c = 0; c < KT; c++) {
+          const uint32_t w = DropStage::word(drop_lds + buf * DropStage::BYTES, 32 * gq + l32, c) >> (4 * g);
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int32_t sel = __builtin_amdgcn_sbfe((int)w, 8 * (r >> 2) + (r & 3), 1);   // keep ? ~0 : 0
+            p[c][r] = __uint_as_float(__float_as_uint(p[c][r]) & (uint32_t)sel);        // (1 / keep_prob: once, on O)
+          }
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < KT; c++)
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++) {
+          typename E::V2 t0 = E::cvt2(p[c][8 * hh + 0], p[c][8 * hh + 1]);
+          typename E::V2 t1 = E::cvt2(p[c][8 * hh + 2], p[c][8 * hh + 3]);
+          typename E::V2 t2 = E::cvt2(p[c][8 * hh + 4], p[c][8 * hh + 5]);
+          typename E::V2 t3 = E::cvt2(p[c][8 * hh + 6], p[c][8 * hh + 7]);
+          V8 pv = {t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+          pf[gq][c][hh] = pv;
+        }
+      if (__any(alpha != 1.0f)) {
+#pragma unroll
+        for (int db = 0; db < C::DB; db++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) o[gq][db][r] *= alpha;
+      }
+    }
+  };
+
   if (j_lo <= j_hi) {
     tile_dma<T, D, BN, NW>(kp, a.k_ss, j_lo * BN, a.Sk, smem);
     tile_dma<T, D, BN, NW>(vp, a.v_ss, j_lo * BN, a.Sk, smem + TILEB);
@@ -143,235 +356,29 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
     // it places no vmcnt wait inside the loop -- such a wait would also stall on the next tile's DMA.
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-
-#ifdef ACCT_TRACE
-#define TR(k) if (blockIdx.x == ACCT_TRACE && lane == 0 && j - j_lo < 48) ((unsigned long long*)(a.lse + (size_t)a.B * a.N * a.Sq))[((wave * 48) + (j - j_lo)) * 8 + (k)] = __builtin_amdgcn_s_memtime()
-#else
-#define TR(k)
-#endif
-    // block classes of a dense mask: 64 blocks at a time into scalar registers
-    const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
-    BlkClassWindow flwin;
-    flwin.init(flrow, 1, j_lo / TPB, j_hi / TPB, lane);
     for (int j = j_lo; j <= j_hi; j++) {
-      TR(0);
-      const uint32_t fl_cur = flwin.get(j / TPB, lane);
       const int buf = (j - j_lo) & 1;
       ACCT_LDS char* kbuf = smem + buf * 2 * TILEB;
       ACCT_LDS char* vbuf = kbuf + TILEB;
       if (j < j_hi) {                                       // next tile streams into the other buffer meanwhile
         ACCT_LDS char* nb = smem + (buf ^ 1) * 2 * TILEB;
-        if ((j + 2) * BN <= a.Sk) {
-          kdma.issue(kp, a.k_ss, (j + 1) * BN, nb);
-          vdma.issue(vp, a.v_ss, (j + 1) * BN, nb + TILEB);
-        } else {                                            // ragged last tile: clamped rows
-          tile_dma<T, D, BN, NW>(kp, a.k_ss, (j + 1) * BN, a.Sk, nb);
-          tile_dma<T, D, BN, NW>(vp, a.v_ss, (j + 1) * BN, a.Sk, nb + TILEB);
-        }
+        stage_tile(kdma, kp, a.k_ss, j + 1, nb);
+        stage_tile(vdma, vp, a.v_ss, j + 1, nb + TILEB);
         DropStage::issue(a, bh, wq0, j + 1, lane, drop_lds + (buf ^ 1) * DropStage::BYTES);
       }
-      const int kv0 = j * BN;
-      const int kvb = j / TPB;
-      bool act = (kvb - a.next_blk <= wqb) && (wqb <= kvb + a.prev_blk) && (wq0 < a.Sq);
-      if (causal) act = act && (kv0 <= wq_end - 1);
-      act = act && (kv0 < wkv_limit);
-      bool apply_mask = false;
-      bool diag = causal;                                   // keys after the query are hidden, by index compare
-      if (MASKT && a.mask_kind == kMaskDense && act) {
-        act = fl_cur != kBlkSkip;
-        apply_mask = fl_cur == kBlkApply;
-        if (fl_cur == kBlkTriu) { diag = true; act = kv0 <= wq_end - 1; }
-      } else if (MASKT && a.mask_kind == kMaskTile) {
-        apply_mask = wqb == kvb;
-      }
-      TR(1);
-      if (act) {
-        // ---- S^T = K Q^T : s[gq][c] is the 32(kv) x 32(q) tile of kv chunk c ----
+      const uint32_t info = classify(j);
+      if (info & kAct) {
         f32x16 s[QG][KT];
-#pragma unroll
-        for (int gq = 0; gq < QG; gq++)
-#pragma unroll
-          for (int c = 0; c < KT; c++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) s[gq][c][r] = 0.f;
-        if constexpr (KT == 2) {
-          V8 kf[2][C::KS];                                  // every K fragment of the tile is requested up front;
-#pragma unroll                                              // the MFMAs then start as the reads return in order
-          for (int c = 0; c < 2; c++)
-#pragma unroll
-            for (int t = 0; t < C::KS; t++) kf[c][t] = lds_read_frag<T>(kbuf + koff[t] + c * 32 * C::PITCH);
-#pragma unroll
-          for (int c = 0; c < 2; c++)
-#pragma unroll
-            for (int t = 0; t < C::KS; t++)
-#pragma unroll
-              for (int gq = 0; gq < QG; gq++) s[gq][c] = E::mfma(kf[c][t], qf[gq][t], s[gq][c]);
-        } else {
-#pragma unroll
-          for (int c = 0; c < KT; c++)
-#pragma unroll
-            for (int t = 0; t < C::KS; t++) {
-              const V8 kf = lds_read_frag<T>(kbuf + koff[t] + c * 32 * C::PITCH);
-#pragma unroll
-              for (int gq = 0; gq < QG; gq++) s[gq][c] = E::mfma(kf, qf[gq][t], s[gq][c]);
-            }
-        }
-        TR(2);
-        // element (gq, c, r): q = wq0 + 32 gq + l32 ; kv = kv0 + 32 c + 8 (r/4) + 4 g + r%4
-        const bool edge = apply_mask || (diag && (kv0 + BN - 1 > wq0)) || (kv0 + BN > a.Sk);
-        typename E::V8 pf[QG][KT][2];
-#pragma unroll
-        for (int gq = 0; gq < QG; gq++) {
-          const int qrow = wq0 + 32 * gq + l32;
-          const int qrow_c = min(qrow, a.Sq - 1);            // clamped for side-input addressing
-          if (BIAS) {
-            if (bias_staged) {
-              typename E::V4 bv[2][4];
-#pragma unroll
-              for (int c = 0; c < 2; c++)
-#pragma unroll
-                for (int r4 = 0; r4 < 4; r4++) bv[c][r4] = bias_tile_read<T>(bias_lds + gq * 4096, l32, 4 * c + r4, g);
-              if (gq == QG - 1) {
-                // the tile is in registers: its LDS region can take the next tile, which has the rest of
-                // this step to land (the end-of-step wait covers it)
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                if (j < j_hi) stage_bias(j + 1);
-              }
-#pragma unroll
-              for (int c = 0; c < 2; c++)
-#pragma unroll
-                for (int r4 = 0; r4 < 4; r4++)
-#pragma unroll
-                  for (int e = 0; e < 4; e++)
-                    s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale, (float)bv[c][r4][e]);
-            } else {
-#pragma unroll
-              for (int c = 0; c < 2; c++)
-#pragma unroll
-                for (int r4 = 0; r4 < 4; r4++) {
-                  const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
-                  float bias[4];
-                  load_bias4<T>(alibip + (int64_t)qrow_c * a.al_sq, kv, a.Sk, alibi_vec, bias);
-#pragma unroll
-                  for (int e = 0; e < 4; e++)
-                    s[gq][c][4 * r4 + e] = __builtin_fmaf(s[gq][c][4 * r4 + e], a.scale, bias[e]);
-                }
-            }
-          }
-          if (edge) {
-            if (apply_mask) {
-#pragma unroll
-              for (int c = 0; c < KT; c++)
-#pragma unroll
-                for (int r4 = 0; r4 < 4; r4++) {
-                  const int kv = kv0 + 32 * c + 8 * r4 + 4 * g;
-                  uint32_t mbits;
-                  if (a.mask_kind == kMaskDense) mbits = load_u8x4(maskp + (int64_t)qrow_c * a.Sk, kv, a.Sk, mask_vec);
-                  else mbits = load_u8x4(maskp + (qrow_c & 127) * 128, kv & 127, 128, mask_vec);
-#pragma unroll
-                  for (int e = 0; e < 4; e++)
-                    if ((mbits >> (8 * e)) & 0xffu) s[gq][c][4 * r4 + e] += madd;
-                }
-            }
-            if (diag && kv0 + BN - 1 > wq0 + 32 * gq) {
-              // Keys after the query are removed outright: with the additive mask their probability
-              // underflows to exactly 0 as well (the diagonal key is always visible), so the result
-              // is the same bit for bit at a third of the vector instructions.
-              const int dl = qrow - kv0 - 4 * g;
-#pragma unroll
-              for (int c = 0; c < KT; c++)
-#pragma unroll
-                for (int r = 0; r < 16; r++)
-                  if (32 * c + 8 * (r >> 2) + (r & 3) > dl) s[gq][c][r] = -INFINITY;
-            }
-            if (kv0 + BN > a.Sk) {                             // ragged key tail
-              const int lim = a.Sk - kv0 - 4 * g;
-#pragma unroll
-              for (int c = 0; c < KT; c++)
-#pragma unroll
-                for (int r = 0; r < 16; r++)
-                  if (32 * c + 8 * (r >> 2) + (r & 3) >= lim) s[gq][c][r] = -INFINITY;
-            }
-          }
-          // ---- online softmax for query row qrow ----
-          float mx = s[gq][0][0];
-#pragma unroll
-          for (int c = 0; c < KT; c++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[gq][c][r]);
-          mx = pair_max(mx);
-          // Lazy running max: it only moves when a score beats it by more than 2^8 in probability
-          // terms.  Until then P = exp2(s - m) may reach 256 instead of 1 (harmless in fp16/bf16 and in
-          // the fp32 sums; O = acc / l and LSE = m + ln l are unchanged), and the O rescale below is
-          // skipped for almost every tile after the first.
-          const bool grow = mx > m[gq] + lazy_thr;
-          const float m_new = grow ? mx : m[gq];
-          const float alpha = grow ? fast_exp2((m[gq] - m_new) * cmul) : 1.0f;
-          const float mc = m_new * cmul;
-          m[gq] = m_new;
-          float rs = 0.f;
-          float p[KT][16];
-#pragma unroll
-          for (int c = 0; c < KT; c++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-              p[c][r] = fast_exp2(__builtin_fmaf(s[gq][c][r], cmul, -mc));
-              rs += p[c][r];
-            }
-          lsum[gq] = lsum[gq] * alpha + rs;                  // row sum BEFORE dropout
-          if (DROP) {
-            // keep bits of this row and tile: word c covers keys kv0 + 32c .. +31
-#pragma unroll
-            for (int c = 0; c < KT; c++) {
-              const uint32_t w = DropStage::word(drop_lds + buf * DropStage::BYTES, 32 * gq + l32, c) >> (4 * g);
-#pragma unroll
-              for (int r = 0; r < 16; r++) {
-                const int32_t sel = __builtin_amdgcn_sbfe((int)w, 8 * (r >> 2) + (r & 3), 1);   // keep ? ~0 : 0
-                p[c][r] = __uint_as_float(__float_as_uint(p[c][r]) & (uint32_t)sel);        // (1 / keep_prob: once, on O)
-              }
-            }
-          }
-#pragma unroll
-          for (int c = 0; c < KT; c++)
-#pragma unroll
-            for (int hh = 0; hh < 2; hh++) {
-              typename E::V2 t0 = E::cvt2(p[c][8 * hh + 0], p[c][8 * hh + 1]);
-              typename E::V2 t1 = E::cvt2(p[c][8 * hh + 2], p[c][8 * hh + 3]);
-              typename E::V2 t2 = E::cvt2(p[c][8 * hh + 4], p[c][8 * hh + 5]);
-              typename E::V2 t3 = E::cvt2(p[c][8 * hh + 6], p[c][8 * hh + 7]);
-              V8 pv = {t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
-              pf[gq][c][hh] = pv;
-            }
-          if (__any(alpha != 1.0f)) {
-#pragma unroll
-            for (int db = 0; db < C::DB; db++)
-#pragma unroll
-              for (int r = 0; r < 16; r++) o[gq][db][r] *= alpha;
-          }
-        }
-        TR(3);
-        // ---- O^T += V^T P^T ----
-#pragma unroll
-        for (int c = 0; c < KT; c++)
-#pragma unroll
-          for (int hh = 0; hh < 2; hh++)
-#pragma unroll
-            for (int db = 0; db < C::DB; db++) {
-              const ACCT_LDS char* vaddr = vbuf + voff[db] + (32 * c + 16 * hh) * C::PITCH;
-              const V8 vf = join_tr<T>(lds_read_tr(vaddr), lds_read_tr(vaddr + C::tr_hi(db)));
-#pragma unroll
-              for (int gq = 0; gq < QG; gq++) o[gq][db] = E::mfma(vf, pf[gq][c][hh], o[gq][db]);
-            }
+        V8 pf[QG][KT][2];
+        gemm_s(kbuf, s);
+        softmax(j, buf, info, s, pf);
+        gemm_pv(vbuf, pf);
       } else if (BIAS && bias_staged && j < j_hi && wq0 < a.Sq) {
         stage_bias(j + 1);                                  // nothing to read in this step: the region is free
       }
-      TR(4);
       dma_wait();
-      TR(5);
       __syncthreads();
-      TR(6);
     }
-#undef TR
   }
 
   // ---- epilogue: O = O^T / l, LSE = m + ln l.  Each wave transposes its rows through its own
@@ -425,7 +432,7 @@ static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
   const size_t tiles = 4 * 32 * KT * (size_t)C::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0) + (size_t)NW * 2 * DropRowStage<DROP, QG, KT>::BYTES, stage = (size_t)NW * 32 * (C::DB * 64 + 16);
   const size_t smem = tiles > stage ? tiles : stage;
   auto kern = mask_t ? fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, true, KT> : fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, BIAS || DROP, KT>;
-  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  hipError_t e = allow_dynamic_lds((const void*)kern, smem);
   if (e != hipSuccess) return e;
   const long long nblk = (long long)a.n_tiles * a.B * a.N;
   hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(64 * NW), smem, st, a);
@@ -446,11 +453,10 @@ static hipError_t launch_fwd_q(const FaArgs& a, hipStream_t st) {
   return launch_fwd_t<T, D, QG, NW, false, false>(a, st);
 }
 
-// variant: 1 = 4 waves x 32 rows, 2 = 4 waves x 64 rows, 3 = 8 waves x 32 rows
+// variant: 1 = 4 waves x 32 rows, 3 = 8 waves x 32 rows
 template <typename T, int D>
 static hipError_t launch_fwd_d(const FaArgs& a, int variant, hipStream_t st) {
-  if (variant == 3) return launch_fwd_q<T, D, 1, 8>(a, st);
-  return variant == 2 ? launch_fwd_q<T, D, 2, 4>(a, st) : launch_fwd_q<T, D, 1, 4>(a, st);
+  return variant == 3 ? launch_fwd_q<T, D, 1, 8>(a, st) : launch_fwd_q<T, D, 1, 4>(a, st);
 }
 // head dims 40 and 160: 32 rows per wave only
 template <typename T, int D>

@@ -2,9 +2,27 @@
 #pragma once
 #include "fa_common.hpp"
 
+#include <mutex>
+#include <set>
+#include <utility>
+
 namespace acct {
 
-// forward: qg = query groups of 32 rows per wave (1 or 2); the bias / dropout
+// Raises a kernel's dynamic LDS limit once per (kernel, device) instead of on every launch.
+inline hipError_t allow_dynamic_lds(const void* kern, size_t bytes) {
+  static std::mutex mu;
+  static std::set<std::pair<const void*, int>> done;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  std::lock_guard<std::mutex> lock(mu);
+  if (done.count({kern, dev})) return hipSuccess;
+  e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e == hipSuccess) done.insert({kern, dev});
+  return e;
+}
+
+// forward: variant 3 = 8 waves x 32 query rows, 1 = 4 waves x 32 rows; the bias / dropout
 // variants are picked from a.alibi / a.droprow
 hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st);
 

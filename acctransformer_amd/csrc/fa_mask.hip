@@ -1,4 +1,5 @@
-// Block classification of a dense uint8 attention mask.
+// Block classification of a dense attention mask (uint8, or the I/O dtype as the reference passes it;
+// nonzero = masked either way).
 //
 // The reference adds -10000 to masked scores (attention.py:357-371 of the
 // reference's flash_attention ops) instead of removing them.  A 128x128 block
@@ -22,11 +23,12 @@ constexpr uint8_t kBlkAllMasked = 255;  // provisional: resolved to skip or appl
 // t/8 of every 128x128 block, so a block is one 16-byte load per thread and many blocks are in
 // flight at once.  Per-block "any masked" / "any unmasked" bits are gathered in two 64-bit masks
 // and reduced once at the end.
+template <int ES>
 __global__ void __launch_bounds__(1024) fa_mask_blocks_vec_kernel(const FaArgs a, uint8_t* flags) {
   __shared__ unsigned long long s_m, s_u;
   const int qb = blockIdx.x % a.Tr, mb = blockIdx.x / a.Tr;
   const int tid = threadIdx.x, row = qb * 128 + (tid >> 3), c0 = (tid & 7) * 16;
-  const uint8_t* mrow = a.mask + (int64_t)mb * a.mask_sb + (int64_t)min(row, a.Sq - 1) * a.Sk;
+  const uint8_t* mrow = a.mask + ((int64_t)mb * a.mask_sb + (int64_t)min(row, a.Sq - 1) * a.Sk) * ES;
   uint8_t* frow = flags + ((int64_t)mb * a.Tr + qb) * a.Tc;
   int lo = max(0, qb - a.prev_blk), hi = min(a.Tc - 1, qb + a.next_blk);
   if (a.row_prefix) hi = min(hi, ((qb * 128 / a.row_prefix + 1) * a.row_prefix - 1) / 128);
@@ -44,20 +46,33 @@ __global__ void __launch_bounds__(1024) fa_mask_blocks_vec_kernel(const FaArgs a
       for (int i = 0; i < n; i++) {
         const int kv = (base + i) * 128 + c0;
         if (kv < a.Sk) {                                // Sk % 16 == 0: a piece is entirely inside or outside
-          const u32x4 v = *reinterpret_cast<const u32x4*>(mrow + kv);
-          // a byte is zero iff (x - 0x01010101) & ~x & 0x80808080 has its top bit set
           bool has_zero = false, has_nonzero = false;
+          uint32_t nz = 0;                              // bit e: element e of this thread's 16 is nonzero
 #pragma unroll
-          for (int w = 0; w < 4; w++) {
-            has_nonzero |= v[w] != 0;
-            has_zero |= ((v[w] - 0x01010101u) & ~v[w] & 0x80808080u) != 0;
+          for (int h = 0; h < ES; h++) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(mrow + (int64_t)kv * ES + 16 * h);
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+              if (ES == 1) {
+                // a byte is zero iff (x - 0x01010101) & ~x & 0x80808080 has its top bit set
+                has_nonzero |= v[w] != 0;
+                has_zero |= ((v[w] - 0x01010101u) & ~v[w] & 0x80808080u) != 0;
+#pragma unroll
+                for (int e = 0; e < 4; e++) nz |= (((v[w] >> (8 * e)) & 0xffu) != 0 ? 1u : 0u) << (4 * w + e);
+              } else {
+                // 2-byte floating-point elements: the sign of a zero does not count
+                const uint32_t lo16 = v[w] & 0x7fffu, hi16 = (v[w] >> 16) & 0x7fffu;
+                has_nonzero |= (lo16 | hi16) != 0;
+                has_zero |= lo16 == 0 || hi16 == 0;
+                nz |= ((lo16 != 0 ? 1u : 0u) | (hi16 != 0 ? 2u : 0u)) << (8 * h + 2 * w);
+              }
+            }
           }
           if (has_nonzero) bm |= 1ull << i;
           if (has_zero) bu |= 1ull << i;
           if (base + i == qb) {
 #pragma unroll
-            for (int e = 0; e < 16; e++)
-              tri_bad |= (((v[e >> 2] >> (8 * (e & 3))) & 0xffu) != 0) != (c0 + e > (tid >> 3));
+            for (int e = 0; e < 16; e++) tri_bad |= (((nz >> e) & 1u) != 0) != (c0 + e > (tid >> 3));
           }
         }
       }
@@ -90,11 +105,12 @@ __global__ void __launch_bounds__(1024) fa_mask_blocks_vec_kernel(const FaArgs a
 }
 
 // Generic path (any alignment): one workgroup per (mask batch, q block); thread t scans 64 columns of row t/2
+template <int ES>
 __global__ void __launch_bounds__(256) fa_mask_blocks_kernel(const FaArgs a, uint8_t* flags) {
   const int qb = blockIdx.x % a.Tr, mb = blockIdx.x / a.Tr;
   const int tid = threadIdx.x, row = qb * 128 + (tid >> 1), c0 = (tid & 1) * 64;
-  const uint8_t* mrow = a.mask + (int64_t)mb * a.mask_sb + (int64_t)min(row, a.Sq - 1) * a.Sk;
-  const bool vec_ok = (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0;
+  const uint8_t* mrow = a.mask + ((int64_t)mb * a.mask_sb + (int64_t)min(row, a.Sq - 1) * a.Sk) * ES;
+  const bool vec_ok = ((((uintptr_t)a.mask / ES) | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 3) == 0;
   uint8_t* frow = flags + ((int64_t)mb * a.Tr + qb) * a.Tc;
   int lo = max(0, qb - a.prev_blk), hi = min(a.Tc - 1, qb + a.next_blk);
   if (a.row_prefix) hi = min(hi, ((qb * 128 / a.row_prefix + 1) * a.row_prefix - 1) / 128);
@@ -110,7 +126,7 @@ __global__ void __launch_bounds__(256) fa_mask_blocks_kernel(const FaArgs a, uin
         const int kv = kvb * 128 + c0 + c;
         if (kv >= a.Sk) break;
         const int n = min(4, a.Sk - kv);
-        const uint32_t bits = load_u8x4(mrow, kv, a.Sk, vec_ok);
+        const uint32_t bits = load_mask4(mrow, kv, a.Sk, vec_ok, ES);
 #pragma unroll
         for (int e = 0; e < 4; e++)
           if (e < n) {
@@ -138,58 +154,64 @@ __global__ void __launch_bounds__(256) fa_mask_blocks_kernel(const FaArgs a, uin
 // rows of a block packed into 128 bits per key column, so that the kernel reads one 32-bit word per lane
 // and 32-row chunk instead of 16 single bytes.  One thread per key column and word (32 rows): the loads
 // of a thread are independent, and 512 threads keep enough of them in flight.
+template <int ES>
 __global__ void __launch_bounds__(512) fa_mask_colbits_kernel(const FaArgs a, const uint8_t* flags, uint32_t* out) {
   const int kvb = blockIdx.x % a.Tc, qb = (blockIdx.x / a.Tc) % a.Tr, mb = blockIdx.x / (a.Tc * a.Tr);
   if (flags[((int64_t)mb * a.Tr + qb) * a.Tc + kvb] != kBlkApply) return;
   const int kv = kvb * 128 + (threadIdx.x & 127), i = threadIdx.x >> 7;
   if (kv >= a.Sk) return;
-  const uint8_t* col = a.mask + (int64_t)mb * a.mask_sb + kv;
+  const uint8_t* col = a.mask + ((int64_t)mb * a.mask_sb + kv) * ES;
   uint32_t w = 0u;
 #pragma unroll
   for (int r = 0; r < 32; r++) {
     const int row = qb * 128 + 32 * i + r;
-    if (row < a.Sq && col[(int64_t)row * a.Sk]) w |= 1u << r;
+    if (row < a.Sq && elem_nonzero<ES>(col, (int64_t)row * a.Sk)) w |= 1u << r;
   }
   out[(((int64_t)mb * a.Tr + qb) * a.Sk + kv) * 4 + i] = w;
 }
 
 // the same for the compact 128x128 tile that is applied on diagonal blocks: out[key][4]
+template <int ES>
 __global__ void __launch_bounds__(128) fa_mask_tilebits_kernel(const uint8_t* tile, uint32_t* out) {
   uint32_t w[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
   for (int i = 0; i < 4; i++)
 #pragma unroll 8
     for (int r = 0; r < 32; r++)
-      if (tile[(32 * i + r) * 128 + threadIdx.x]) w[i] |= 1u << r;
+      if (elem_nonzero<ES>(tile, (32 * i + r) * 128 + threadIdx.x)) w[i] |= 1u << r;
   u32x4 v = {w[0], w[1], w[2], w[3]};
   *reinterpret_cast<u32x4*>(out + threadIdx.x * 4) = v;
 }
 
 hipError_t launch_mask_colbits(const FaArgs& a, const uint8_t* flags, uint32_t* out, int MB, hipStream_t st) {
   if (a.mask_kind == kMaskTile) {
-    hipLaunchKernelGGL(fa_mask_tilebits_kernel, dim3(1), dim3(128), 0, st, a.mask, out);
+    if (a.mask_es == 2) hipLaunchKernelGGL(fa_mask_tilebits_kernel<2>, dim3(1), dim3(128), 0, st, a.mask, out);
+    else hipLaunchKernelGGL(fa_mask_tilebits_kernel<1>, dim3(1), dim3(128), 0, st, a.mask, out);
     return hipGetLastError();
   }
-  hipLaunchKernelGGL(fa_mask_colbits_kernel, dim3((unsigned)(MB * a.Tr * a.Tc)), dim3(512), 0, st, a, flags, out);
+  const dim3 grid((unsigned)(MB * a.Tr * a.Tc));
+  if (a.mask_es == 2) hipLaunchKernelGGL(fa_mask_colbits_kernel<2>, grid, dim3(512), 0, st, a, flags, out);
+  else hipLaunchKernelGGL(fa_mask_colbits_kernel<1>, grid, dim3(512), 0, st, a, flags, out);
   return hipGetLastError();
 }
 
-// Dropout mask (uint8, nonzero = keep) packed into keep bits, by query row for the kernels whose lanes own
+// Dropout mask (uint8 {0,1}, or the reference's {0, 1/keep_prob} in the I/O dtype; nonzero = keep) packed into keep bits, by query row for the kernels whose lanes own
 // query rows (forward, dQ) and by key column for the dK/dV kernel.  One wave per (batch*head, 128 query
 // rows, 1024 keys): per row every lane loads the 16 bytes of keys 16*lane .. +15 (a kilobyte per wave
 // instruction keeps enough bytes in flight) and turns them into 16 bits; lane pairs form the 32-bit row words.
 //   rowbits [B*N*Sq, 2*ceil(Sk/64)] 32-bit: bit k of word w = keep[row][32w + k];
 //   colbits [B*N, Tr, Sk, 4] 32-bit: bit r of the 128-bit entry = keep[128*qb + r][key].
+template <int ES>
 __global__ void __launch_bounds__(64) fa_drop_bits_kernel(const FaArgs a, uint32_t* rowbits, uint32_t* colbits) {
   const int nspan = (a.Sk + 1023) / 1024;
   const int span = blockIdx.x % nspan, qb = (blockIdx.x / nspan) % a.Tr, bh = blockIdx.x / (nspan * a.Tr);
   const int lane = threadIdx.x;
   const int kv = span * 1024 + 16 * lane;               // first of this lane's sixteen keys
-  const bool vec = (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 15) == 0 && kv + 16 <= a.Sk;
+  const bool vec = (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 15) == 0 && kv + 16 <= a.Sk;   // (16 elements: ES aligned 16-byte loads)
   const int widx = 32 * span + (lane >> 1);             // this lane pair's word within the row
   const bool writer = rowbits && (lane & 1) == 0 && widx < a.droprow_w;
   uint32_t* rowout = rowbits + ((int64_t)bh * a.Sq + qb * 128) * a.droprow_w + widx;
-  const uint8_t* p = a.drop + ((int64_t)bh * a.Sq + qb * 128) * a.Sk + min(kv, max(a.Sk - 16, 0));
+  const uint8_t* p = a.drop + (((int64_t)bh * a.Sq + qb * 128) * a.Sk + min(kv, max(a.Sk - 16, 0))) * ES;
   const int nrow = min(128, a.Sq - qb * 128);
   uint32_t cw[16][4];                                   // per key: four words of 32 rows, most significant bit first
 #pragma unroll
@@ -199,24 +221,33 @@ __global__ void __launch_bounds__(64) fa_drop_bits_kernel(const FaArgs a, uint32
 #pragma unroll 4
     for (int r = 0; r < 32; r++) {
       const int rr = 32 * i + r;
-      u32x4 v = {0u, 0u, 0u, 0u};
+      uint32_t nz = 0;                                  // bit e: this lane's key e of the row is kept
       if (rr < nrow) {
-        if (vec) v = *reinterpret_cast<const u32x4*>(p);
-        else {
-          const uint8_t* q = a.drop + ((int64_t)bh * a.Sq + qb * 128 + rr) * a.Sk;
+        if (vec) {
+#pragma unroll
+          for (int h = 0; h < ES; h++) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(p + 16 * h);
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+              if (ES == 1) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) nz |= (((v[w] >> (8 * e)) & 0xffu) != 0 ? 1u : 0u) << (4 * w + e);
+              } else {
+                nz |= (((v[w] & 0x7fffu) != 0 ? 1u : 0u) | (((v[w] >> 16) & 0x7fffu) != 0 ? 2u : 0u)) << (8 * h + 2 * w);
+              }
+            }
+          }
+        } else {
+          const uint8_t* q = a.drop + ((int64_t)bh * a.Sq + qb * 128 + rr) * a.Sk * ES;
 #pragma unroll
           for (int e = 0; e < 16; e++)
-            if (kv + e < a.Sk) v[e >> 2] |= (uint32_t)q[kv + e] << (8 * (e & 3));
+            if (kv + e < a.Sk && elem_nonzero<ES>(q, kv + e)) nz |= 1u << e;
         }
       }
-      p += a.Sk;                                        // per-lane pointer walks down the rows
-      uint32_t bits = 0;
+      p += (int64_t)a.Sk * ES;                          // per-lane pointer walks down the rows
+      const uint32_t bits = nz;
 #pragma unroll
-      for (int e = 0; e < 16; e++) {
-        const uint32_t keep = ((v[e >> 2] >> (8 * (e & 3))) & 0xffu) != 0 ? 1u : 0u;
-        bits |= keep << e;
-        cw[e][i] = (cw[e][i] << 1) | keep;
-      }
+      for (int e = 0; e < 16; e++) cw[e][i] = (cw[e][i] << 1) | ((nz >> e) & 1u);
       uint32_t x = bits << (16 * (lane & 1));
       x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xf, 0xf, true);    // lane ^ 1
       if (writer && rr < nrow) *rowout = x;
@@ -291,14 +322,22 @@ hipError_t launch_drop_philox(const FaArgs& a, uint32_t* rowbits, uint32_t* colb
 
 hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st) {
   const long long nblk = (long long)a.B * a.N * a.Tr * ((a.Sk + 1023) / 1024);
-  hipLaunchKernelGGL(fa_drop_bits_kernel, dim3((unsigned)nblk), dim3(64), 0, st, a, rowbits, colbits);
+  if (a.drop_es == 2) hipLaunchKernelGGL(fa_drop_bits_kernel<2>, dim3((unsigned)nblk), dim3(64), 0, st, a, rowbits, colbits);
+  else hipLaunchKernelGGL(fa_drop_bits_kernel<1>, dim3((unsigned)nblk), dim3(64), 0, st, a, rowbits, colbits);
   return hipGetLastError();
 }
 
 hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, int MB, hipStream_t st) {
+  // fast path: every 16-element piece of a row is 16-byte aligned and entirely inside or outside the row
   const bool vec = (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 15) == 0;
-  if (vec) hipLaunchKernelGGL(fa_mask_blocks_vec_kernel, dim3((unsigned)(MB * a.Tr)), dim3(1024), 0, st, a, flags);
-  else hipLaunchKernelGGL(fa_mask_blocks_kernel, dim3((unsigned)(MB * a.Tr)), dim3(256), 0, st, a, flags);
+  const dim3 grid((unsigned)(MB * a.Tr));
+  if (a.mask_es == 2) {
+    if (vec) hipLaunchKernelGGL(fa_mask_blocks_vec_kernel<2>, grid, dim3(1024), 0, st, a, flags);
+    else hipLaunchKernelGGL(fa_mask_blocks_kernel<2>, grid, dim3(256), 0, st, a, flags);
+  } else {
+    if (vec) hipLaunchKernelGGL(fa_mask_blocks_vec_kernel<1>, grid, dim3(1024), 0, st, a, flags);
+    else hipLaunchKernelGGL(fa_mask_blocks_kernel<1>, grid, dim3(256), 0, st, a, flags);
+  }
   return hipGetLastError();
 }
 

@@ -17,6 +17,10 @@ Differences from the reference that a caller can see:
     as "nonzero = masked" (the reference multiplies its value by -10000, and
     only ever feeds 0/1).  A floating dropout_mask is the reference's
     {0, 1/keep_prob} form; a uint8/bool one is {0,1} with `keep_prob` given.
+    Masks in q's dtype (the reference's form) and uint8 masks are handed to
+    the library as they are, without a conversion pass; other dtypes are
+    converted to uint8 first.  Without `keep_prob`, a floating dropout mask
+    costs one reduction and a host sync to recover keep_prob = 1 / max.
   * `dropout_mask` may also be a `(seed, offset)` pair of ints: the keep mask
     is then drawn inside the library (Philox4x32-10, defined in
     include/acct_fa.h) instead of being read from a [B,N,Sq,Sk] tensor, the
@@ -55,42 +59,50 @@ def _is_compact_shape(shape):
     return False
 
 
-def _classify_mask(attn_mask, Sq, Sk):
-    """Returns (mask_kind, uint8 tensor or None).  The outcome is remembered per
-    tensor object and version, so a mask reused across steps is inspected once."""
+DETECT_CAUSAL_MASKS = True     # look once per mask tensor whether it is the plain causal mask (one device compare, one sync)
+
+
+def _classify_mask(attn_mask, Sq, Sk, io_dtype):
+    """Returns (mask_kind, tensor or None).  A mask in the operands' dtype -- the
+    reference's form -- or in uint8 goes to the library as it is; only other
+    dtypes are converted.  The outcome is remembered per tensor object and
+    version, so a mask reused across steps is inspected once."""
     key = id(attn_mask)
     hit = _mask_cache.get(key)
-    if hit is not None and hit[0]() is attn_mask and hit[1] == attn_mask._version and hit[2] == (Sq, Sk):
+    if hit is not None and hit[0]() is attn_mask and hit[1] == attn_mask._version and hit[2] == (Sq, Sk, io_dtype):
         return hit[3], hit[4]
-    if attn_mask.dtype in (torch.uint8, torch.bool):
-        m8 = attn_mask.contiguous().view(torch.uint8) if attn_mask.dtype == torch.bool else attn_mask.contiguous()
+    if attn_mask.dtype == torch.bool:
+        m = attn_mask.contiguous().view(torch.uint8)
+    elif attn_mask.dtype in (torch.uint8, io_dtype):
+        m = attn_mask.contiguous()
     else:
-        m8 = attn_mask.ne(0).to(torch.uint8)
+        m = attn_mask.ne(0).to(torch.uint8)
+    wide = m.dtype != torch.uint8
     compact = _is_compact_shape(tuple(attn_mask.shape)) and not (Sq == TILING_BLOCK_SIZE and Sk == TILING_BLOCK_SIZE
                                                                   and attn_mask.dim() == 3)
     if compact:
-        tri = torch.triu(torch.ones(128, 128, dtype=torch.uint8, device=m8.device), diagonal=1)
-        if torch.equal(m8.reshape(128, 128), tri):
+        tri = torch.triu(torch.ones(128, 128, dtype=torch.bool, device=m.device), diagonal=1)
+        if torch.equal(m.reshape(128, 128).ne(0), tri):
             kind, out = _capi.MASK_CAUSAL, None      # evaluated by index compare, no loads
         else:
-            kind, out = _capi.MASK_TILE_U8, m8.reshape(128, 128)
+            kind, out = (_capi.MASK_TILE_F16 if wide else _capi.MASK_TILE_U8), m.reshape(128, 128)
         compact_kind = True
     else:
         compact_kind = False
-        if m8.dim() == 2:
-            m8 = m8.unsqueeze(0)
-        if m8.dim() != 3 or m8.shape[1] != Sq or m8.shape[2] != Sk:
+        if m.dim() == 2:
+            m = m.unsqueeze(0)
+        if m.dim() != 3 or m.shape[1] != Sq or m.shape[2] != Sk:
             raise ValueError(f"attn_mask must be [1|B,{Sq},{Sk}] or a (1,128,128) causal tile, got {tuple(attn_mask.shape)}")
-        kind, out = _capi.MASK_DENSE_U8, m8
-        if Sq == Sk:
-            rows = torch.arange(Sq, device=m8.device)
-            tri = (rows[None, :] > rows[:, None]).to(torch.uint8)
-            if all(torch.equal(m8[i], tri) for i in range(m8.shape[0])):
+        kind, out = (_capi.MASK_DENSE_F16 if wide else _capi.MASK_DENSE_U8), m
+        if DETECT_CAUSAL_MASKS and Sq == Sk:
+            rows = torch.arange(Sq, device=m.device)
+            tri = rows[None, :] > rows[:, None]
+            if torch.equal(m.ne(0), tri.expand_as(m)):
                 kind, out = _capi.MASK_CAUSAL, None
     if len(_mask_cache) > 64:
         for k_ in [k_ for k_, v_ in _mask_cache.items() if v_[0]() is None]:
             del _mask_cache[k_]
-    _mask_cache[key] = (weakref.ref(attn_mask), attn_mask._version, (Sq, Sk), kind, out, compact_kind)
+    _mask_cache[key] = (weakref.ref(attn_mask), attn_mask._version, (Sq, Sk, io_dtype), kind, out, compact_kind)
     return kind, out
 
 
@@ -98,8 +110,9 @@ def _is_seed_pair(x):
     return isinstance(x, (tuple, list)) and len(x) == 2 and all(isinstance(t, int) for t in x)
 
 
-def _prepare_dropout(dropout_mask, keep_prob):
-    """Returns (uint8 mask or None, keep_prob, (seed, offset) or None)."""
+def _prepare_dropout(dropout_mask, keep_prob, io_dtype):
+    """Returns (mask or None, keep_prob, (seed, offset) or None).  The mask goes to the library as uint8 {0,1}
+    or, in the operands' dtype, as the reference's {0, 1/keep_prob}."""
     if dropout_mask is None:
         return None, 1.0, None
     if _is_seed_pair(dropout_mask):
@@ -116,18 +129,20 @@ def _prepare_dropout(dropout_mask, keep_prob):
     if keep_prob is None:
         mx = float(dropout_mask.max())
         keep_prob = 1.0 / mx if mx > 0 else 1.0
+    if dropout_mask.dtype == io_dtype:
+        return dropout_mask.contiguous(), float(keep_prob), None
     return dropout_mask.ne(0).to(torch.uint8), float(keep_prob), None
 
 
 def _build_params(q, k, v, attn_mask, dropout_mask, alibi_mask, prev_block_num, next_block_num, scale, keep_prob,
                   row_block_prefix=0):
     Sq, Sk = q.shape[2], k.shape[2]
-    kind, m8 = (_capi.MASK_NONE, None) if attn_mask is None else _classify_mask(attn_mask, Sq, Sk)
+    kind, m8 = (_capi.MASK_NONE, None) if attn_mask is None else _classify_mask(attn_mask, Sq, Sk, q.dtype)
     if kind == _capi.MASK_CAUSAL and attn_mask is not None and _mask_cache[id(attn_mask)][5] and next_block_num > 0:
         # a compact tile only ever touches diagonal blocks (attention.py:363-365,
         # flash_attention_fwd.py:353-356): blocks right of the diagonal stay visible
         kind, m8 = _capi.MASK_TILE_U8, torch.triu(torch.ones(128, 128, dtype=torch.uint8, device=q.device), diagonal=1)
-    d8, keep, seed = _prepare_dropout(dropout_mask, keep_prob)
+    d8, keep, seed = _prepare_dropout(dropout_mask, keep_prob, q.dtype)
     if alibi_mask is not None and alibi_mask.dtype != q.dtype:
         alibi_mask = alibi_mask.to(q.dtype)
     return _capi.make_params(q, k, v, scale=scale, keep_prob=keep, prev_block_num=prev_block_num,

@@ -69,9 +69,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--settle-seconds", type=float, default=0.6,
+                    help="untimed steps run for this long after the warm-up so that the clocks have settled")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the ALiBi and padded-batch + dropout configurations (extra keys of the JSON line)")
     ap.add_argument("--no-dense-pass", action="store_true",
-                    help="skip the untimed dense-mask comparison pass (so that a profile covers the timed workload only)")
+                    help="skip the untimed dense-mask and TriangleAttention comparison passes (so that a profile covers the timed workload only)")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also run an elementwise fp32 copy kernel over this many MiB (5 launches) after the timed "
                          "region: a known-size reference for scaling profiler byte counters")
@@ -134,6 +138,17 @@ def main():
     for _ in range(args.warmup):
         step(p)
     torch.cuda.synchronize()
+    # Clock settle: the first ~100 steps after an idle period run on clocks that are still moving (measured:
+    # up to 16 % slower), whatever --warmup says.  Keep stepping untimed until half a second of work has gone
+    # through the GPU; the timed region below then starts on settled clocks.
+    t_s = time.perf_counter()
+    settle_steps = 0
+    while time.perf_counter() - t_s < args.settle_seconds:
+        for _ in range(20):
+            step(p)
+        torch.cuda.synchronize()
+        settle_steps += 20
+    settle_s = time.perf_counter() - t_s
 
     K = args.steps
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(K)]
@@ -195,6 +210,69 @@ def main():
                "block_skip_speedup": round(ms_all / ms_tri, 3)}
         del qt, kt, vt, mt
 
+    # The other two training configurations (untimed for `value`; extra keys of the line): forward + fused
+    # backward through the C ABI, kernel time by HIP events on the launch stream, algorithmic flops by the same
+    # convention, and the algorithmic HBM bytes per step (every operand read or written once: q, k, v, O, dO,
+    # dQ, dK, dV, LSE twice, and the side inputs once per call that reads them) over the same time.
+    other = None
+    if not args.no_other_configs:
+        other = {}
+
+        def run_config(name, pp, qq, kk, vv, dd, flops, side_bytes, n=10):
+            oo, ll = torch.empty_like(qq), torch.empty(qq.shape[:3], dtype=torch.float32, device=dev)
+            g3 = [torch.empty_like(t) for t in (qq, kk, vv)]
+            pp.o_stride = _capi._bhs_strides(oo)
+            nw = max(lib.acct_fa_bwd_workspace_bytes(P(pp)), lib.acct_fa_fwd_workspace_bytes(P(pp)), 256)
+            w = torch.empty(nw, dtype=torch.uint8, device=dev)
+
+            def one():
+                check(lib.acct_fa_fwd(P(pp), oo.data_ptr(), ll.data_ptr(), w.data_ptr(), nw, st))
+                check(lib.acct_fa_bwd(P(pp), oo.data_ptr(), dd.data_ptr(), ll.data_ptr(), g3[0].data_ptr(), g3[1].data_ptr(),
+                                      g3[2].data_ptr(), w.data_ptr(), nw, st))
+            for _ in range(3):
+                one()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(n):
+                one()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / n
+            io = 8 * qq.numel() * qq.element_size() + 2 * ll.numel() * 4 + side_bytes
+            other[name] = {"ms_per_step": round(ms, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
+                           "algorithmic_hbm_gb_per_step": round(io / 1e9, 3), "achieved_hbm_gbps": round(io / (ms * 1e-3) / 1e9, 1),
+                           "hbm_peak_gbps": 8000.0}
+
+        # ALiBi + causal, B2 N32 S4096 D128: bias -slope_h (i - j), as a full [1,N,S,S] tensor and in the
+        # reference's row-bias form [1,N,1,S] (slope_h j: the row constant cancels in the softmax)
+        B3, N3, S3 = 2, 32, 4096
+        q3, k3, v3, d3 = (torch.randn(B3, N3, S3, D, generator=g).half().to(dev) for _ in range(4))
+        slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / N3) for h in range(N3)], device=dev)
+        pos = torch.arange(S3, device=dev, dtype=torch.float32)
+        al_row = (slopes[None, :, None, None] * pos[None, None, None, :]).half()
+        al_full = (-slopes[None, :, None, None] * (pos[None, None, :, None] - pos[None, None, None, :])).half()
+        fl3 = 14.0 * B3 * N3 * S3 * S3 * D * 0.5
+        for nm, al in (("alibi_causal_B2_N32_S4096_row_bias", al_row), ("alibi_causal_B2_N32_S4096_full_bias", al_full)):
+            pp = _capi.make_params(q3, k3, v3, scale=scale, next_block_num=0, mask_kind=_capi.MASK_CAUSAL, alibi=al)
+            run_config(nm, pp, q3, k3, v3, d3, fl3, 2 * al.numel() * 2)      # the bias is read by the forward and by the backward
+        del q3, k3, v3, d3, al_row, al_full
+        # padded batch + dropout, B16 N16 S1024 D128: key-padding mask [B,S,S] uint8, lengths U[256,1024]; dropout
+        # mask uint8 [B,N,S,S] Bernoulli(0.9)
+        B5, N5, S5 = 16, 16, 1024
+        q5, k5, v5, d5 = (torch.randn(B5, N5, S5, D, generator=g).half().to(dev) for _ in range(4))
+        lens = torch.randint(256, S5 + 1, (B5,), generator=g)
+        m5 = (torch.arange(S5)[None, None, :] >= lens[:, None, None]).expand(B5, S5, S5).to(torch.uint8).contiguous().to(dev)
+        dr5 = (torch.rand(B5, N5, S5, S5, generator=g) < 0.9).to(torch.uint8).to(dev)
+        f5 = float(lens.float().mean()) / S5
+        fl5 = 14.0 * B5 * N5 * S5 * S5 * D * f5
+        pp = _capi.make_params(q5, k5, v5, scale=scale, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m5, drop_mask=dr5)
+        run_config("padded_dropout_B16_N16_S1024_mask_tensor", pp, q5, k5, v5, d5, fl5, 2 * (m5.numel() + dr5.numel()))
+        pp = _capi.make_params(q5, k5, v5, scale=scale, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m5, drop_seed=1234)
+        run_config("padded_dropout_B16_N16_S1024_seed_pair", pp, q5, k5, v5, d5, fl5, 2 * m5.numel())
+        other["padded_dropout_unmasked_fraction"] = round(f5, 4)
+        del q5, k5, v5, d5, m5, dr5
+
     if args.calib_copy_mib > 0:
         src = torch.ones(args.calib_copy_mib * (1 << 18), dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
@@ -235,6 +313,8 @@ def main():
         "fwd_tflops": round(fl_fwd / (t_fwd * 1e-3) / 1e12, 1), "bwd_tflops": round(fl_bwd / ((t_dq + t_dkdv) * 1e-3) / 1e12, 1),
         "dense_mask_path_ms_per_step": None if ms_dense is None else round(ms_dense, 4),
         "triangle_block_skip": tri,
+        "other_configs": other,
+        "clock_settle": {"seconds": round(settle_s, 3), "steps": settle_steps},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": traffic_bytes[dom]},
     }

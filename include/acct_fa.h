@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define ACCT_FA_VERSION 103
+#define ACCT_FA_VERSION 104
 
 /* error codes (0 = success) */
 #define ACCT_OK          0
@@ -49,9 +49,19 @@ extern "C" {
 /* attn_mask interpretation */
 #define ACCT_MASK_NONE     0
 #define ACCT_MASK_DENSE_U8 1   /* uint8 [1|B, Sq, Sk], nonzero = masked (adds -10000); T/attention.py:357-371 */
+#define ACCT_MASK_DENSE_F16 2  /* the same mask in p->dtype (fp16 / bf16), the form the reference op takes
+                                  (T/flash_attention_impl.py:43-45, T/attention.py:270-277,357-371): nonzero = masked.
+                                  The reference multiplies the mask VALUE by -10000 and only ever feeds 0 / 1. */
 #define ACCT_MASK_TILE_U8  3   /* uint8 [128,128] tile applied only where q_blk == kv_blk:
                                   the reference's compact causal mode, T/attention.py:279-285,363-365 */
 #define ACCT_MASK_CAUSAL   4   /* no tensor: -10000 added where j > i, evaluated by index compare */
+#define ACCT_MASK_TILE_F16 5   /* the compact [128,128] tile in p->dtype (the reference's own form of it) */
+
+/* drop_mask interpretation (drop_mask_kind) */
+#define ACCT_DROP_U8  0        /* uint8 [B,N,Sq,Sk] of {0,1}, nonzero = keep */
+#define ACCT_DROP_F16 1        /* p->dtype [B,N,Sq,Sk] of {0, 1/keep_prob}, the form the reference op takes
+                                  (T/flash_attention_impl.py:48-55, T/attention.py:373-395): nonzero = keep; the
+                                  scaling comes from keep_prob, which the caller still passes */
 
 #define ACCT_BLOCK_UNBOUNDED 65536   /* default prev/next_block_num, L/flash_attention.py:95-96 */
 
@@ -84,8 +94,8 @@ typedef struct acct_fa_params {
   const void*    q;
   const void*    k;
   const void*    v;
-  const uint8_t* attn_mask;      /* per mask_kind; NULL when NONE / CAUSAL */
-  const uint8_t* drop_mask;      /* uint8 [B,N,Sq,Sk] of {0,1}, contiguous; NULL = no dropout */
+  const void*    attn_mask;      /* per mask_kind, contiguous; NULL when NONE / CAUSAL */
+  const void*    drop_mask;      /* per drop_mask_kind, [B,N,Sq,Sk] contiguous; NULL = no dropout */
   const void*    alibi;          /* dtype, see strides; NULL = none (T/attention.py:347-355) */
   /* Counter-based dropout (fields added in version 101): with drop_philox != 0, drop_mask == NULL and
      keep_prob < 1 the keep mask is never materialised by the caller -- the library derives it from
@@ -112,7 +122,7 @@ typedef struct acct_fa_params {
      (drop_seed, drop_offset, keep_prob) and on B, N, Sq, Sk only. */
   void*    drop_bits;
   int32_t  drop_bits_filled;
-  int32_t  reserved0;
+  int32_t  drop_mask_kind;       /* ACCT_DROP_* (field added in version 104; 0 = the uint8 form) */
 } acct_fa_params;
 
 /* Forward: replaces the `flash_attention` TBE custom op, T/flash_attention_fwd.py:498-530

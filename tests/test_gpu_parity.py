@@ -331,6 +331,15 @@ def test_block_band(prev, nxt):
     _check_all(q, k, v, dO, okw, _run(q, k, v, dO, scale=D ** -0.5, prev=prev, nxt=nxt))
 
 
+@pytest.mark.parametrize("D", [64, 80])
+def test_bf16_backward_at_the_small_head_dims(D):
+    B, N, S = 2, 2, 300
+    q, k, v, dO = (_gen((B, N, S, D), s, torch.bfloat16) for s in (136, 137, 138, 139))
+    tri = np.triu(np.ones((1, S, S), np.uint8), 1)
+    _check_all(q, k, v, dO, dict(scale=D ** -0.5, attn_mask=tri),
+               _run(q, k, v, dO, scale=D ** -0.5, mask_kind=_capi.MASK_CAUSAL), ATOL_BF16, RTOL_BF16)
+
+
 def test_bf16_io():
     B, N, S, D = 2, 2, 512, 128
     q, k, v, dO = (_gen((B, N, S, D), s, torch.bfloat16) for s in (36, 37, 38, 39))
@@ -347,10 +356,34 @@ def test_strided_bsnd_inputs():
     p = _capi.make_params(q, k, v, scale=D ** -0.5, mask_kind=_capi.MASK_CAUSAL)
     o, lse = _capi.fa_fwd(p, q)
     assert o.stride() == q.stride()
-    grads = _capi.fa_bwd(p, q, k, v, o, dO.contiguous().as_strided(o.size(), o.stride()) if False else dO, lse)
+    grads = _capi.fa_bwd(p, q, k, v, o, dO, lse)
     torch.cuda.synchronize()
     tri = np.triu(np.ones((1, S, S), np.uint8), 1)
     _check_all(q, k, v, dO, dict(scale=D ** -0.5, attn_mask=tri), (o, lse, grads))
+    # an upstream gradient whose strides differ from O's (contiguous BNSD against the permuted O) is copied
+    # element by element into O's layout, not relabelled
+    grads_c = _capi.fa_bwd(p, q, k, v, o, dO.contiguous(), lse)
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(grads, grads_c))
+
+
+def test_strided_inputs_through_autograd_with_contiguous_upstream_gradient():
+    # autograd does not promise grad_output in O's strides: (o * w).sum() with a contiguous w hands a contiguous dO
+    B, N, S, D = 2, 3, 200, 64
+    base = [_gen((B, S, N, D), s) for s in (140, 141, 142)]
+    q, k, v = (t.to(DEV).permute(0, 2, 1, 3).requires_grad_(True) for t in base)
+    w = _gen((B, N, S, D), 143).to(DEV)
+    fa = get_flash_attention(scale=D ** -0.5)
+    o, lse = fa(q, k, v)
+    assert not o.is_contiguous()
+    (o.float() * w.float()).sum().backward()
+    torch.cuda.synchronize()
+    qn, kn, vn = (_np(t) for t in (q, k, v))
+    O, _ = orc.unfused_fwd(qn, kn, vn, scale=D ** -0.5)
+    _gate(O, o, what="O")
+    dQ, dK, dV = orc.unfused_bwd(qn, kn, vn, _np(w), scale=D ** -0.5)
+    for name, ref, got in (("dQ", dQ, q.grad), ("dK", dK, k.grad), ("dV", dV, v.grad)):
+        _gate(ref, got, what=name)
 
 
 # ---- slice equivalence and determinism (ST/test_sharding.py:19-115) ---------------
@@ -674,10 +707,196 @@ def test_split_backward_entry_points_match_fused_call():
     assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
 
 
+# ---- the reference's own mask forms at the C boundary (masks in the operands' dtype) ---------------
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_reference_form_masks_equal_the_uint8_forms_bit_for_bit(dtype):
+    # attn_mask in q's dtype with 1 = masked (flash_attention_impl.py:43-45 of the reference ops) and dropout
+    # mask in q's dtype with values {0, 1/keep_prob} (:48-55), read by the library without a conversion pass
+    B, N, Sq, Sk, D = 2, 3, 300, 333, 128
+    q, k, v, dO = (_gen(sh, s, dtype) for sh, s in (((B, N, Sq, D), 150), ((B, N, Sk, D), 151), ((B, N, Sk, D), 152), ((B, N, Sq, D), 153)))
+    rng = np.random.default_rng(154)
+    m8 = (rng.random((B, Sq, Sk)) < 0.3).astype(np.uint8)
+    m8[:, :, 250:] = 1                                        # a fully masked tail (skipped blocks) ...
+    m8[:, :, :100] = 0                                        # ... and clean blocks in front
+    d8 = (rng.random((B, N, Sq, Sk)) < 0.8).astype(np.uint8)
+    keep = 0.8
+    mf = torch.from_numpy(m8).to(dtype)
+    mf[0, 5, 7] = -0.0                                        # a negative zero is a zero: -0 * -10000 adds nothing
+    m8[0, 5, 7] = 0
+    df = (torch.from_numpy(d8).float() / keep).to(dtype)
+    scale = D ** -0.5
+    ref = _run(q, k, v, dO, scale=scale, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m8, drop_mask=d8, keep_prob=keep)
+    got = _run(q, k, v, dO, scale=scale, mask_kind=_capi.MASK_DENSE_F16, attn_mask=mf, drop_mask=df, keep_prob=keep)
+    assert torch.equal(ref[0], got[0]) and torch.equal(ref[1], got[1])
+    assert all(torch.equal(a, b) for a, b in zip(ref[2], got[2]))
+    tol = (ATOL, RTOL) if dtype == torch.float16 else (ATOL_BF16, RTOL_BF16)
+    _check_all(q, k, v, dO, dict(scale=scale, attn_mask=m8, drop_mask=d8, keep_prob=keep), got, *tol)
+
+
+def test_reference_form_masks_on_aligned_shapes_and_compact_tile():
+    # 16-byte aligned rows take the vector pre-passes; the compact (1,128,128) tile in fp16 is the reference's own form
+    B, N, S, D = 2, 2, 512, 128
+    q, k, v, dO = (_gen((B, N, S, D), s) for s in (155, 156, 157, 158))
+    lens = [384, 200]
+    m8 = np.zeros((B, S, S), np.uint8)
+    for b, n in enumerate(lens):
+        m8[b, :, n:] = 1
+    m8 |= np.triu(np.ones((S, S), np.uint8), 1)[None]
+    d8 = (np.random.default_rng(159).random((B, N, S, S)) < 0.9).astype(np.uint8)
+    mf, df = torch.from_numpy(m8).half(), (torch.from_numpy(d8).float() / 0.9).half()
+    scale = D ** -0.5
+    ref = _run(q, k, v, dO, scale=scale, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m8, drop_mask=d8, keep_prob=0.9)
+    got = _run(q, k, v, dO, scale=scale, mask_kind=_capi.MASK_DENSE_F16, attn_mask=mf, drop_mask=df, keep_prob=0.9)
+    assert torch.equal(ref[0], got[0]) and all(torch.equal(a, b) for a, b in zip(ref[2], got[2]))
+    _check_all(q, k, v, dO, dict(scale=scale, attn_mask=m8, drop_mask=d8, keep_prob=0.9), got)
+    tile8 = np.triu(np.ones((128, 128), np.uint8), 1)
+    tile8[3, 1] = 1
+    ref = _run(q, k, v, dO, scale=scale, mask_kind=_capi.MASK_TILE_U8, attn_mask=tile8, nxt=0)
+    got = _run(q, k, v, dO, scale=scale, mask_kind=_capi.MASK_TILE_F16, attn_mask=torch.from_numpy(tile8).half(), nxt=0)
+    assert torch.equal(ref[0], got[0]) and all(torch.equal(a, b) for a, b in zip(ref[2], got[2]))
+
+
+def test_operator_takes_reference_form_masks_without_conversion():
+    # through the Python operator: an fp16 padding mask and an fp16 {0, 1/keep_prob} dropout mask, keep_prob recovered
+    B, N, S, D = 2, 2, 256, 128
+    q, k, v, dO = (_gen((B, N, S, D), s) for s in (160, 161, 162, 163))
+    m8 = np.zeros((B, S, S), np.uint8); m8[0, :, 200:] = 1; m8[1, :, 130:] = 1
+    d8 = (np.random.default_rng(164).random((B, N, S, S)) < 0.75).astype(np.uint8)
+    fa = get_flash_attention(scale=D ** -0.5)
+    qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    o, lse = fa(qd, kd, vd, torch.from_numpy(m8).half().to(DEV), (torch.from_numpy(d8).float() / 0.75).half().to(DEV))
+    o.backward(dO.to(DEV))
+    torch.cuda.synchronize()
+    _check_all(q, k, v, dO, dict(scale=D ** -0.5, attn_mask=m8, drop_mask=d8, keep_prob=0.75), (o, lse, (qd.grad, kd.grad, vd.grad)))
+
+
+# ---- the reference's CPU-sized configuration through the HIP path ------------------------------------
+def test_cpu_sized_configuration_b1_n4_s512_d64():
+    # B=1, N=4, S=512, D=64, scale 1/8, no mask, forward: against the fp64 operator spec and against the
+    # reference's own CPU path (numpy fp16 unfused attention, tests/train/flash_attention/st/common.py:110-132),
+    # which takes the scale folded into q
+    B, N, S, D = 1, 4, 512, 64
+    rng = np.random.default_rng(1000)
+    q, k, v = (rng.standard_normal((B, N, S, D)).astype(np.float16) for _ in range(3))
+    o, lse, _ = _run(q, k, v, scale=0.125)
+    O, L = orc.unfused_fwd(q.astype(np.float32), k.astype(np.float32), v.astype(np.float32), scale=0.125)
+    _gate(O, o, what="O vs fp64 spec")
+    assert np.max(np.abs(L - _np(lse))) < 1e-4
+    qs = (q.astype(np.float32) * 0.125).astype(np.float16)          # exact: a power of two
+    O16, _mid = orc.np_unfused_fwd_fp16(qs, k, v)
+    # the reference's fp16 pipeline rounds scores and probabilities to fp16: its own tolerance applies
+    verdict, over, over_max = orc.data_compare(O16.astype(np.float32), _np(o))
+    assert verdict == "Pass", (over, over_max)
+
+
+# ---- both branches of the workgroup map (more / not more than 64 batch*head pairs) -------------------
+def test_slice_equivalence_across_the_workgroup_map_branches():
+    # B*N = 256 takes the XCD-grouped launch order, each slice of 64 the plain one: every (batch, head) pair must
+    # come out bit for bit the same either way (tests/train/flash_attention/st/test_sharding.py:19-81 design).
+    # (S = 1024 keeps a slice at 256 workgroups, so that the slices run the same kernel variant as the whole.)
+    B, N, S, D = 8, 32, 1024, 128
+    q, k, v, dO = (_gen((B, N, S, D), s) for s in (170, 171, 172, 173))
+    kw = dict(scale=D ** -0.5, mask_kind=_capi.MASK_CAUSAL, nxt=0)
+    o, lse, g = _run(q, k, v, dO, **kw)
+    for b0 in range(0, B, 2):
+        sl = slice(b0, b0 + 2)
+        o_s, lse_s, g_s = _run(q[sl], k[sl], v[sl], dO[sl], **kw)
+        assert torch.equal(o[sl], o_s) and torch.equal(lse[sl], lse_s)
+        assert all(torch.equal(a[sl], b_) for a, b_ in zip(g, g_s))
+
+
+# ---- the reference's long-sequence shapes at full length ---------------------------------------------
+@pytest.mark.parametrize("q_len, kv_len", [(256, 128 * 1024), (128 * 1024, 256)])
+def test_reference_long_sequence_shapes_without_mask(q_len, kv_len):
+    # tests/train/flash_attention/st/test_fa_fwd_precision.py:70-94: (1,1,256,128) x (1,1,131072,128) and its
+    # mirror, uniform [0,1) inputs, the raw operator (scale 1), no mask
+    D = 128
+    rng = np.random.default_rng(180)
+    q = rng.random((1, 1, q_len, D)).astype(np.float16)
+    k = rng.random((1, 1, kv_len, D)).astype(np.float16)
+    v = rng.random((1, 1, kv_len, D)).astype(np.float16)
+    dO = rng.standard_normal((1, 1, q_len, D)).astype(np.float16)
+    o, lse, grads = _run(q, k, v, dO, scale=1.0)
+    O, L = orc.unfused_fwd(q.astype(np.float32), k.astype(np.float32), v.astype(np.float32), scale=1.0)
+    _gate(O, o, what="O")
+    assert orc.data_compare(O, _np(o))[0] == "Pass"
+    assert np.max(np.abs(L - _np(lse))) < 1e-4 * max(1.0, np.abs(L).max() / 10)
+    # backward (the reference tests these shapes forward only): with all-positive keys dQ = sum_j dS_ij k_j carries
+    # the rounding of the saved O through D = rowsum(dO*O) at full weight, so the ground truth takes D from the
+    # rounded forward output, as the reference's own does (tests/train/flash_attention/st/common.py:156-169)
+    ref = orc.unfused_bwd(q.astype(np.float32), k.astype(np.float32), v.astype(np.float32), dO.astype(np.float32), scale=1.0,
+                          O_saved=_np(o))
+    _gate(ref[0], grads[0], what="dQ")
+    if q_len <= kv_len:
+        _gate(ref[1], grads[1], what="dK")
+        _gate(ref[2], grads[2], what="dV")
+    else:
+        # dK and dV of a key are sums over 131072 query rows of products whose 16-bit operand (P, dS) is rounded to
+        # fp16 before the MFMA; with these inputs a few keys hold most of the probability mass of every row, and
+        # the rounding alone moves their sums by more than the gate.  The bar here: the kernel stays within three
+        # times the error of exact sums over fp16-rounded P and dS (the rounding any fp16 kernel of this
+        # formulation performs), plus the gate.
+        qd, kd, vd, dd, od = (x[0, 0].astype(np.float64) for x in (q, k, v, dO, _np(o)))
+        sc = qd @ kd.T
+        P = np.exp(sc - sc.max(-1, keepdims=True)); P /= P.sum(-1, keepdims=True)
+        dS = P * (dd @ vd.T - (dd * od).sum(-1, keepdims=True))
+        r16 = lambda x: x.astype(np.float16).astype(np.float64)
+        e_dk = np.abs(r16(dS).T @ qd - dS.T @ qd).max()
+        e_dv = np.abs(r16(P).T @ dd - P.T @ dd).max()
+        for name, r, g_, e in (("dK", ref[1], grads[1], e_dk), ("dV", ref[2], grads[2], e_dv)):
+            ok, ratio, mx = orc.tolerance_gate(r, _np(g_), atol=ATOL + 3 * e, rtol=RTOL)
+            assert ok, f"{name}: worst ratio {ratio:.3f}, max |d| {mx:.3e}, fp16 operand rounding alone {e:.3e}"
+
+
+def test_reference_flash_vs_triangle_attention_at_32k():
+    # tests/train/flash_attention/st/test_fa_fwd_precision.py:97-120: FlashAttention with a [B,S,S] fp16 causal mask
+    # against TriangleAttention with block size 1024 at S = 32768 (4 of the reference's 40 heads: the kernels
+    # index by (batch, head) pair alike); uniform [0,1) inputs
+    B, N, S, D = 1, 4, 32 * 1024, 128
+    g = torch.Generator().manual_seed(181)
+    q, k, v = (torch.rand((B, N, S, D), generator=g).half().to(DEV) for _ in range(3))
+    mask = torch.triu(torch.ones(S, S, dtype=torch.float16, device=DEV), 1).unsqueeze(0)       # 2 GiB on the device
+    p = _capi.make_params(q, k, v, scale=1.0, mask_kind=_capi.MASK_DENSE_F16, attn_mask=mask)
+    o_fa, lse_fa = _capi.fa_fwd(p, q)
+    tri = TriangleAttention(block_size=1024).eval()
+    o_tri = tri(q, k, v, mask)
+    torch.cuda.synchronize()
+    verdict, over, over_max = orc.data_compare(_np(o_tri), _np(o_fa))
+    assert verdict == "Pass", (over, over_max)
+    assert torch.allclose(o_fa.float(), o_tri.float(), atol=2e-3, rtol=1e-3)
+    # a sample of query rows against the fp64 spec over the whole key range
+    rows = np.array([0, 1, 127, 128, 1023, 1024, 16383, 16384, 32767])
+    mrows = (np.arange(S)[None, :] > rows[:, None]).astype(np.uint8)[None]
+    for h in (0, N - 1):
+        O, L = orc.unfused_fwd(_np(q[:, h:h + 1, rows]), _np(k[:, h:h + 1]), _np(v[:, h:h + 1]), scale=1.0, attn_mask=mrows)
+        _gate(O, o_fa[:, h:h + 1, rows], what="O rows")
+        assert np.max(np.abs(L - _np(lse_fa[:, h:h + 1, rows]))) < 1e-4 * 3
+
+
 # ---- the benchmark configurations at full size -------------------------------------
 def _sample_heads(B, N, n=3, seed=0):
     rng = np.random.default_rng(seed)
     return sorted({(int(rng.integers(B)), int(rng.integers(N))) for _ in range(n)} | {(B - 1, N - 1)})
+
+
+def _torch_cpu_causal_attention(q, k, v, dO, scale):
+    """Every (batch, head) pair in torch fp32 on the host cores (a second formulation: additive -10000 mask,
+    torch softmax, autograd for the gradients).  The callers gate it against the fp64 oracle on sampled heads
+    before they use it for all heads."""
+    B, N, S, D = q.shape
+    add = torch.triu(torch.full((S, S), -10000.0), 1)
+    outs = []
+    for b in range(B):
+        qf, kf, vf = (t[b].float().requires_grad_(dO is not None) for t in (q, k, v))
+        sc = torch.matmul(qf, kf.transpose(-1, -2)) * scale + add
+        O = torch.matmul(torch.softmax(sc, -1), vf)
+        L = torch.logsumexp(sc, -1)
+        if dO is not None:
+            O.backward(dO[b].float())
+            outs.append((O.detach(), L.detach(), qf.grad, kf.grad, vf.grad))
+        else:
+            outs.append((O.detach(), L.detach()))
+    return [torch.stack([o[i] for o in outs]).numpy() for i in range(len(outs[0]))]
 
 
 def test_full_size_fa2_causal_fwd_bwd():
@@ -688,10 +907,21 @@ def test_full_size_fa2_causal_fwd_bwd():
     scale = D ** -0.5
     o, lse, g = _run(q, k, v, dO, scale=scale, mask_kind=_capi.MASK_DENSE_U8, attn_mask=tri, nxt=0)
     oc, lsec, gc = _run(q, k, v, dO, scale=scale, mask_kind=_capi.MASK_CAUSAL, nxt=0)
+    # every head: against torch fp32 on the host, which is itself held to the fp64 oracle on the sampled heads
+    # (at a tenth of the gate) so that the two together pin all 64 (batch, head) pairs
+    tO, tL, tdQ, tdK, tdV = _torch_cpu_causal_attention(q, k, v, dO, scale)
     for b, h in _sample_heads(B, N):
         sl = (slice(b, b + 1), slice(h, h + 1))
         _check_all(q[sl], k[sl], v[sl], dO[sl], dict(scale=scale, attn_mask=tri),
                    (o[sl], lse[sl], tuple(t[sl] for t in g)))
+        O, L = orc.unfused_fwd(_np(q[sl]), _np(k[sl]), _np(v[sl]), scale=scale, attn_mask=tri)
+        grads = orc.unfused_bwd(_np(q[sl]), _np(k[sl]), _np(v[sl]), _np(dO[sl]), scale=scale, attn_mask=tri)
+        for ref, tt in zip((O,) + tuple(grads), (tO, tdQ, tdK, tdV)):
+            assert orc.tolerance_gate(ref, tt[sl], atol=2e-4, rtol=1e-4)[0]
+        assert np.max(np.abs(L - tL[sl])) < 1e-4
+    for name, ref, got in (("O", tO, o), ("dQ", tdQ, g[0]), ("dK", tdK, g[1]), ("dV", tdV, g[2])):
+        _gate(ref, got, 2.2e-3, 1.1e-3, what=name + " (all heads)")
+    assert np.max(np.abs(tL - _np(lse))) < 2e-4
     # the dense-mask path and the index-compare path agree: same blocks, same arithmetic up to the order of
     # the online-softmax steps (the two paths stream keys in tiles of 64 and of 128), i.e. to an fp16 ulp
     close = lambda x, y: torch.allclose(x.float(), y.float(), atol=1e-3, rtol=2e-3)
@@ -730,11 +960,17 @@ def test_full_size_triangle_block_skip():
     o_skip, lse_skip, _ = _run(q, k, v, scale=1.0, mask_kind=_capi.MASK_DENSE_U8, attn_mask=tri, prefix=128)
     o_full, lse_full, _ = _run(q, k, v, scale=1.0, mask_kind=_capi.MASK_DENSE_U8, attn_mask=tri)
     assert torch.equal(o_skip, o_full) and torch.equal(lse_skip, lse_full)     # skipping is exact
+    # all 256 (batch, head) pairs (the XCD-grouped launch order) against torch fp32 on the host, which is held
+    # to the fp64 oracle on the sampled heads
+    tO, tL = _torch_cpu_causal_attention(q, k, v, None, 1.0)
     for b, h in _sample_heads(B, N, n=2, seed=2):
         sl = (slice(b, b + 1), slice(h, h + 1))
         O, L = orc.unfused_fwd(_np(q[sl]), _np(k[sl]), _np(v[sl]), scale=1.0, attn_mask=tri)
         _gate(O, o_skip[sl])
         assert np.max(np.abs(L - _np(lse_skip[sl]))) < 1e-4
+        assert orc.tolerance_gate(O, tO[sl], atol=2e-4, rtol=1e-4)[0] and np.max(np.abs(L - tL[sl])) < 1e-4
+    _gate(tO, o_skip, 2.2e-3, 1.1e-3, what="O (all heads)")
+    assert np.max(np.abs(tL - _np(lse_skip))) < 2e-4
 
 
 def test_full_size_varlen_dropout():

@@ -62,7 +62,8 @@ def _params(**over):
 
 @pytest.mark.parametrize("over, code", [
     (dict(dtype=7), -3), (dict(B=0), -2), (dict(D=512), -4), (dict(D=96), -4), (dict(scale=0.0), -8),
-    (dict(keep_prob=1.5), -8), (dict(prev_block_num=-1), -8), (dict(mask_kind=2), -8),
+    (dict(keep_prob=1.5), -8), (dict(prev_block_num=-1), -8), (dict(mask_kind=6), -8), (dict(mask_kind=_capi.MASK_DENSE_F16), -1),
+    (dict(drop_mask_kind=2), -8),
     (dict(mask_kind=_capi.MASK_DENSE_U8), -1), (dict(row_block_prefix=100), -8), (dict(q=None), -1),
 ])
 def test_validation_error_codes(over, code):
@@ -185,36 +186,45 @@ def test_op_factories_keep_reference_signature():
 
 def test_mask_classification():
     S = 256
-    tri = torch.triu(torch.ones(1, S, S, dtype=torch.float16), 1)
-    assert impl._classify_mask(tri, S, S)[0] == _capi.MASK_CAUSAL
+    f16 = torch.float16
+    tri = torch.triu(torch.ones(1, S, S, dtype=f16), 1)
+    assert impl._classify_mask(tri, S, S, f16)[0] == _capi.MASK_CAUSAL
     pad = torch.zeros(2, S, S, dtype=torch.uint8); pad[:, :, 200:] = 1
-    kind, m8 = impl._classify_mask(pad, S, S)
+    kind, m8 = impl._classify_mask(pad, S, S, f16)
     assert kind == _capi.MASK_DENSE_U8 and m8.dtype == torch.uint8 and m8.shape == (2, S, S)
-    tile = torch.triu(torch.ones(1, 128, 128, dtype=torch.float16), 1)
-    assert impl._classify_mask(tile, S, S)[0] == _capi.MASK_CAUSAL
+    tile = torch.triu(torch.ones(1, 128, 128, dtype=f16), 1)
+    assert impl._classify_mask(tile, S, S, f16)[0] == _capi.MASK_CAUSAL
     odd = tile.clone(); odd[0, 5, 3] = 1
-    kind, m8 = impl._classify_mask(odd, S, S)
-    assert kind == _capi.MASK_TILE_U8 and m8.shape == (128, 128)
-    # remembered per tensor and version: an in-place edit is seen
+    kind, m = impl._classify_mask(odd, S, S, f16)
+    assert kind == _capi.MASK_TILE_F16 and m.shape == (128, 128) and m.dtype == f16     # the reference's form, as it is
+    kind, m = impl._classify_mask(odd.float(), S, S, f16)
+    assert kind == _capi.MASK_TILE_U8 and m.dtype == torch.uint8                        # other dtypes are converted
+    # remembered per tensor and version: an in-place edit is seen; a mask in the operands' dtype is not converted
     tri[0, 0, 1] = 0
-    assert impl._classify_mask(tri, S, S)[0] == _capi.MASK_DENSE_U8
+    kind, m = impl._classify_mask(tri, S, S, f16)
+    assert kind == _capi.MASK_DENSE_F16 and m.data_ptr() == tri.data_ptr()
+    kind, m = impl._classify_mask(tri, S, S, torch.bfloat16)
+    assert kind == _capi.MASK_DENSE_U8 and m.dtype == torch.uint8
     with pytest.raises(ValueError):
-        impl._classify_mask(torch.zeros(1, 100, S), S, S)
+        impl._classify_mask(torch.zeros(1, 100, S), S, S, f16)
 
 
 def test_dropout_mask_forms():
-    d = torch.tensor([[0.0, 1.25], [1.25, 0.0]], dtype=torch.float16)
-    m8, keep, seed = impl._prepare_dropout(d, None)
-    assert m8.tolist() == [[0, 1], [1, 0]] and np.isclose(keep, 0.8) and seed is None
-    m8, keep, seed = impl._prepare_dropout(torch.tensor([[1, 0]], dtype=torch.uint8), 0.9)
+    f16 = torch.float16
+    d = torch.tensor([[0.0, 1.25], [1.25, 0.0]], dtype=f16)
+    m, keep, seed = impl._prepare_dropout(d, None, f16)
+    assert m.data_ptr() == d.data_ptr() and np.isclose(keep, 0.8) and seed is None       # the reference's form, as it is
+    m8, keep, seed = impl._prepare_dropout(d, None, torch.bfloat16)
+    assert m8.tolist() == [[0, 1], [1, 0]] and m8.dtype == torch.uint8 and np.isclose(keep, 0.8)
+    m8, keep, seed = impl._prepare_dropout(torch.tensor([[1, 0]], dtype=torch.uint8), 0.9, f16)
     assert keep == 0.9 and seed is None
     with pytest.raises(ValueError):
-        impl._prepare_dropout(torch.tensor([[1, 0]], dtype=torch.uint8), None)
+        impl._prepare_dropout(torch.tensor([[1, 0]], dtype=torch.uint8), None, f16)
     # a (seed, offset) pair asks the library to draw the mask itself
-    m8, keep, seed = impl._prepare_dropout((1234, 5), 0.75)
+    m8, keep, seed = impl._prepare_dropout((1234, 5), 0.75, f16)
     assert m8 is None and keep == 0.75 and seed == (1234, 5)
     with pytest.raises(ValueError):
-        impl._prepare_dropout((1234, 5), None)
+        impl._prepare_dropout((1234, 5), None, f16)
 
 
 def test_counter_based_dropout_fields_and_workspace():
