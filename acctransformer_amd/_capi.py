@@ -73,6 +73,8 @@ def load():
     lib.acct_fa_fwd.restype = ctypes.c_int
     lib.acct_fa_bwd.argtypes = [P] + [ctypes.c_void_p] * 7 + [ctypes.c_size_t, ctypes.c_void_p]
     lib.acct_fa_bwd.restype = ctypes.c_int
+    lib.acct_fa_bwd_static.argtypes = [P] + [ctypes.c_void_p] * 7
+    lib.acct_fa_bwd_static.restype = ctypes.c_int
     lib.acct_fa_bwd_dq.argtypes = [P] + [ctypes.c_void_p] * 5 + [ctypes.c_size_t, ctypes.c_void_p]
     lib.acct_fa_bwd_dq.restype = ctypes.c_int
     lib.acct_fa_bwd_dkdv.argtypes = [P] + [ctypes.c_void_p] * 6 + [ctypes.c_size_t, ctypes.c_void_p]

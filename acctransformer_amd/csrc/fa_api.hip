@@ -24,6 +24,11 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+// Scratch memory of acct_fa_bwd_static: one copy per GPU the library runs on, held until the process ends.
+// In host code the array's name is only a stand-in: its address on a device comes from
+// hipGetSymbolAddress (static_scratch() below) and nothing else may be passed to a kernel.
+static __device__ __align__(256) unsigned char g_static_scratch[ACCT_FA_STATIC_SCRATCH_BYTES];
+
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_dev_state[kMaxDevices];   // 0 unknown, 1 gfx950, 2 other
 std::atomic<int> g_dev_cus[kMaxDevices];
@@ -42,6 +47,23 @@ int check_device(int* n_cu) {
   }
   if (st != 1) return fail(ACCT_E_ARCH, "device %d is not gfx950; this library carries gfx950 code only", dev);
   *n_cu = g_dev_cus[dev].load(std::memory_order_relaxed);
+  return ACCT_OK;
+}
+
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Address of the current device's copy of g_static_scratch (looked up once per device, with that device current).
+int static_scratch(void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(ACCT_E_ARCH, "no HIP device is current");
+  if (dev < 0 || dev >= kMaxDevices) return fail(ACCT_E_ARCH, "device ordinal %d out of range", dev);
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch));
+    if (e != hipSuccess || !ptr) return fail(ACCT_E_LAUNCH, "hipGetSymbolAddress(static scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
   return ACCT_OK;
 }
 
@@ -318,6 +340,21 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
 int acct_fa_bwd(const acct_fa_params* p, const void* O, const void* dO, const float* LSE, void* dQ, void* dK, void* dV,
                 void* workspace, size_t workspace_bytes, void* stream) {
   return bwd_impl(p, O, dO, LSE, dQ, dK, dV, workspace, workspace_bytes, stream, acct::kStageDq | acct::kStageDkDv);
+}
+
+int acct_fa_bwd_static(const acct_fa_params* p, const void* O, const void* dO, const float* LSE, void* dQ, void* dK, void* dV,
+                       void* stream) {
+  g_err[0] = 0;
+  int rc = validate(p, true);
+  if (rc) return rc;
+  const size_t need = acct_fa_bwd_workspace_bytes(p);
+  if (need > (size_t)ACCT_FA_STATIC_SCRATCH_BYTES)
+    return fail(ACCT_E_WORKSPACE, "acct_fa_bwd_static: this problem needs %zu bytes of scratch, the built-in buffer holds %zu; "
+                "use acct_fa_bwd with a caller-owned workspace", need, (size_t)ACCT_FA_STATIC_SCRATCH_BYTES);
+  void* scratch = nullptr;
+  rc = static_scratch(&scratch);
+  if (rc) return rc;
+  return bwd_impl(p, O, dO, LSE, dQ, dK, dV, scratch, (size_t)ACCT_FA_STATIC_SCRATCH_BYTES, stream, acct::kStageDq | acct::kStageDkDv);
 }
 
 int acct_fa_bwd_dq(const acct_fa_params* p, const void* O, const void* dO, const float* LSE, void* dQ,

@@ -159,6 +159,20 @@ int acct_fa_bwd_dq(const acct_fa_params* p, const void* O, const void* dO, const
 int acct_fa_bwd_dkdv(const acct_fa_params* p, const void* O, const void* dO, const float* LSE,
                      void* dK, void* dV, void* workspace, size_t workspace_bytes, void* stream);
 
+/* acct_fa_bwd for callers that cannot allocate or pass a workspace (code under HIP graph capture, serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as acct_fa_bwd,
+ * bit for bit, minus the workspace: D = rowsum(dO*O), the exp2 offsets, the mask block classes and bitmaps and
+ * the dropout keep bits go to a buffer of ACCT_FA_STATIC_SCRATCH_BYTES that is part of the library's device
+ * image (each GPU the library runs on holds one copy until the process ends).  The call allocates nothing and
+ * frees nothing.  A problem whose acct_fa_bwd_workspace_bytes(p) exceeds the buffer is refused with
+ * ACCT_E_WORKSPACE (pass drop_bits to keep a large dropout mask's bits out of it).  All calls on one GPU share
+ * the buffer: calls that may overlap on that GPU (different streams, different threads) race and must be
+ * serialised by the caller; calls in one stream are ordered and safe.  Nothing in the buffer needs clearing
+ * between calls: every region a call reads is written by that call first. */
+#define ACCT_FA_STATIC_SCRATCH_BYTES (8u << 20)
+int acct_fa_bwd_static(const acct_fa_params* p, const void* O, const void* dO, const float* LSE,
+                       void* dQ, void* dK, void* dV, void* stream);
+
 /* Shape function of the inference operator `FlashAttentionTik` (y = softmax(q k^T) v, no mask, no scale),
  * replacing FlashAttentionTikInferShape, infer/flash_attention/tik/op_proto/flash_attention_tik.cpp:160-193:
  * q, k, v are [batch*heads, seq, D] or [batch, heads, seq, D] (HOST arrays of extents); batch and
