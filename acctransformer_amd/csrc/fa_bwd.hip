@@ -38,7 +38,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   constexpr int BM = 32 * QG * NW;
   constexpr int TILEB = 64 * C::PITCH;
   constexpr int FRING = 4, TRING = 3;                     // fragment reads in flight ahead of their MFMA (row-major / transposed)
-  constexpr bool RINGS = !(BIAS || DROP);                 // (the side-input variants have no registers for the rings)   // fragment reads in flight ahead of their MFMA (row-major / transposed)
+  constexpr bool RINGS = !(BIAS || DROP) && D <= 128;     // (the side-input variants and the wide head dims have no registers for the rings)   // fragment reads in flight ahead of their MFMA (row-major / transposed)
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 buffers][K tile | V tile]; reused by the epilogue
 
@@ -90,9 +90,15 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
     float part = 0.f;
 #pragma unroll
     for (int t = 0; t < C::KS; t++) {
-      qf[gq][t] = *reinterpret_cast<const V8*>(qp + (int64_t)row_c * a.q_ss + 16 * t + 8 * g);
-      dof[gq][t] = *reinterpret_cast<const V8*>(dop + (int64_t)row_c * a.o_ss + 16 * t + 8 * g);
-      const V8 ov = *reinterpret_cast<const V8*>(op + (int64_t)row_c * a.o_ss + 16 * t + 8 * g);
+      // D % 16 == 8: the upper half of the last k-step lies past the row; zeros there make the products
+      // ignore whatever the K / V tiles hold in that slot
+      const bool inside = (D % 16 == 0) || 16 * t + 8 * g < D;
+      V8 z;
+#pragma unroll
+      for (int e = 0; e < 8; e++) z[e] = 0;
+      qf[gq][t] = inside ? *reinterpret_cast<const V8*>(qp + (int64_t)row_c * a.q_ss + 16 * t + 8 * g) : z;
+      dof[gq][t] = inside ? *reinterpret_cast<const V8*>(dop + (int64_t)row_c * a.o_ss + 16 * t + 8 * g) : z;
+      const V8 ov = inside ? *reinterpret_cast<const V8*>(op + (int64_t)row_c * a.o_ss + 16 * t + 8 * g) : z;
 #pragma unroll
       for (int e = 0; e < 8; e++) part += (float)dof[gq][t][e] * (float)ov[e];
     }
@@ -418,22 +424,26 @@ constexpr int kPark = 6;        // stationary fragments parked in LDS per wave (
 constexpr int kParkHot = 4;     // the variant without side inputs has registers for two more fragments
 // stationary fragments parked in LDS per wave: the bias variants give one up for the bias tiles' LDS
 template <int D, bool BIAS, bool MASKT>
-constexpr int dkdv_park() { return D >= 128 ? (BIAS ? kPark - 1 : (MASKT ? kPark : kParkHot)) : 0; }
+constexpr int dkdv_park() { return D == 128 ? (BIAS ? kPark - 1 : (MASKT ? kPark : kParkHot)) : 0; }
+// key groups of 32 rows per wave: head dims above 128 leave registers for the accumulators of one only
+template <int D> constexpr int dkdv_groups() { return D > 128 ? 1 : 2; }
 
 // MASKT = false compiles the mask-tensor handling out (no mask, or the causal mask by index compare):
 // the hot variant must not carry that code's register pressure.
-template <typename T, int D, bool BIAS, bool DROP, bool MASKT>
+template <typename T, int D, bool BIAS, bool DROP, bool MASKT, int NGK = 2>
 __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
+  static_assert(NGK == 2 || (NGK == 1 && !BIAS && !DROP), "one key group per wave: the plain variants only");
   using E = Elem<T>;
   using V8 = typename E::V8;
   using C = SwzCfg<D>;
   constexpr int NW = 8;
-  constexpr int BNK = 256;                          // key rows per workgroup
+  constexpr int WK = 32 * NGK;                      // key rows per wave pair
+  constexpr int BNK = 4 * WK;                       // key rows per workgroup
   constexpr int TILEB = 64 * C::PITCH;
   constexpr int STATB = 2 * 64 * 4;                 // -LSE*log2(e) and D of the 64 rows of a tile
   constexpr int DROPB = DROP ? 2048 : 0;            // keep bits of the tile's 64 rows for the workgroup's 256 keys: [key][2 chunks] words
   constexpr int STAGEB = 2 * TILEB + STATB + DROPB; // one buffer: Q tile | dO tile | -LSE*log2(e) | D | keep bits
-  constexpr int PXB = 4096;                         // P of one pair and chunk: 64 lanes x 64 bytes
+  constexpr int PXB = 2048 * NGK;                   // P of one pair and chunk: 64 lanes x 32 bytes per key group
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 stage buffers][2 x 4 pair P buffers]
   ACCT_LDS char* pexch = smem + 2 * STAGEB;
@@ -446,7 +456,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   wg_map(blockIdx.x, BH, a.n_tiles, bh, kt);
   const int b = bh / a.N, h = bh % a.N;
   const int k0 = kt * BNK;
-  const int wk0 = k0 + pair * 64;                   // first key row of this pair
+  const int wk0 = k0 + pair * WK;                   // first key row of this pair
   const int k_end = min(k0 + BNK, a.Sk);
 
   const T* qp = (const T*)a.q + b * a.q_sb + h * a.q_sh;
@@ -477,7 +487,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   // The last PARK k-steps of the second key group live in a wave-private LDS slab instead of
   // registers (16 VGPRs at D = 128): that is what lets two waves share a SIMD without spilling.
   constexpr int PARK = dkdv_park<D, BIAS, MASKT>();
-  V8 bf[2][C::KS];
+  V8 bf[NGK][C::KS];
   ACCT_LDS char* park = pexch + 8 * PXB + wave * (PARK * 1024) + lane * 16;
   // bias tile (32 query rows x the pair's 64 keys) of the V-role wave, staged one chunk ahead by DMA
   ACCT_LDS char* bias_lds = pexch + 8 * PXB + 8 * (PARK * 1024) + pair * 4096;
@@ -485,19 +495,25 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     const T* src = krole ? vp : kp;
     const int64_t ss = krole ? a.v_ss : a.k_ss;
 #pragma unroll
-    for (int gk = 0; gk < 2; gk++) {
+    for (int gk = 0; gk < NGK; gk++) {
       const int row = min(wk0 + 32 * gk + l32, a.Sk - 1);
 #pragma unroll
       for (int t = 0; t < C::KS; t++) {
-        const V8 v = *reinterpret_cast<const V8*>(src + (int64_t)row * ss + 16 * t + 8 * g);
+        // D % 16 == 8: the upper half of the last k-step lies past the row; zeros there make the products
+        // ignore whatever the Q / dO tiles hold in that slot
+        const bool inside = (D % 16 == 0) || 16 * t + 8 * g < D;
+        V8 v;
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = 0;
+        if (inside) v = *reinterpret_cast<const V8*>(src + (int64_t)row * ss + 16 * t + 8 * g);
         if (gk == 1 && t >= C::KS - PARK) *reinterpret_cast<ACCT_LDS V8*>(park + (t - (C::KS - PARK)) * 1024) = v;
         else bf[gk][t] = v;
       }
     }
   }
-  f32x16 acc[2][C::DB];                             // dV^T (V role) or dK^T (K role): [d rows, key column l32]
+  f32x16 acc[NGK][C::DB];                             // dV^T (V role) or dK^T (K role): [d rows, key column l32]
 #pragma unroll
-  for (int gk = 0; gk < 2; gk++)
+  for (int gk = 0; gk < NGK; gk++)
 #pragma unroll
     for (int db = 0; db < C::DB; db++)
 #pragma unroll
@@ -558,7 +574,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     } else if (MASKT && a.mask_kind == kMaskTile) {
       apply_mask = wkb == qb;
     }
-    const bool limits = (diag && (wk0 + 63 > qc0)) || (wk0 + 64 > a.Sk) || (qc0 + 32 > a.Sq);
+    const bool limits = (diag && (wk0 + WK - 1 > qc0)) || (wk0 + WK > a.Sk) || (qc0 + 32 > a.Sq);
     return (act ? 1u : 0u) | (apply_mask ? 2u : 0u) | (limits ? 4u : 0u) | (diag ? 8u : 0u);
   };
 
@@ -627,7 +643,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
           const ACCT_LDS float* dbuf = lbuf + 64;
           ACCT_LDS char* px = pexch + ((cidx & 1) * 4 + pair) * PXB + ln * 16;
           // rows of this lane's C registers: q = qc0 + 8 (r/4) + 4 g + r%4 ; key = wk0 + 32 gk + l32
-          f32x16 t0[2];                               // S (V role) or dP (K role) of the two key groups
+          f32x16 t0[NGK];                              // S (V role) or dP (K role) of the two key groups
           if (BIAS && bias_staged) {
             // V role: the bias enters as the initial value of the score accumulators (bias / scale, the MFMAs
             // add q.k): no bias registers alive next to the scores.  Transposed reads of the row-major tile:
@@ -635,7 +651,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
             // covers 4 rows x 16 keys and supplies the addresses of that block's 8-byte pieces)
             const ACCT_LDS char* bl = bias_lds + (4 * g + ((lane & 15) >> 2)) * 128 + ((lane >> 4) & 1) * 32 + (lane & 3) * 8;
 #pragma unroll
-            for (int gk = 0; gk < 2; gk++)
+            for (int gk = 0; gk < NGK; gk++)
 #pragma unroll
               for (int i = 0; i < 4; i++) {
                 const typename E::V4 bv = __builtin_bit_cast(typename E::V4, lds_read_tr(bl + i * 8 * 128 + gk * 64));
@@ -644,7 +660,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
               }
           } else {
 #pragma unroll
-            for (int gk = 0; gk < 2; gk++)
+            for (int gk = 0; gk < NGK; gk++)
 #pragma unroll
               for (int r = 0; r < 16; r++) t0[gk][r] = 0.f;
           }
@@ -657,15 +673,15 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
             V8 ar[ARING];
 #pragma unroll
             for (int t = 0; t < ARING; t++) ar[t] = lds_read_frag<T>(abuf + FOFF(t));
-            V8 b1 = (0 >= C::KS - PARK) ? *reinterpret_cast<const ACCT_LDS V8*>(park) : bf[1][0];
+            V8 b1 = (0 >= C::KS - PARK) ? *reinterpret_cast<const ACCT_LDS V8*>(park) : bf[NGK - 1][0];
 #pragma unroll
             for (int t = 0; t < C::KS; t++) {
               V8 b1n = b1;
               if (t + 1 < C::KS)
-                b1n = (t + 1 >= C::KS - PARK) ? *reinterpret_cast<const ACCT_LDS V8*>(park + (t + 1 - (C::KS - PARK)) * 1024) : bf[1][t + 1];
+                b1n = (t + 1 >= C::KS - PARK) ? *reinterpret_cast<const ACCT_LDS V8*>(park + (t + 1 - (C::KS - PARK)) * 1024) : bf[NGK - 1][t + 1];
               __builtin_amdgcn_sched_barrier(0);
               t0[0] = E::mfma(ar[t % ARING], bf[0][t], t0[0]);                              // S[q, key] or dP[q, key]
-              t0[1] = E::mfma(ar[t % ARING], b1, t0[1]);
+              if (NGK == 2) t0[NGK - 1] = E::mfma(ar[t % ARING], b1, t0[NGK - 1]);
               __builtin_amdgcn_sched_barrier(0);
               if (t + ARING < C::KS) ar[t % ARING] = lds_read_frag<T>(abuf + FOFF(t + ARING));
               b1 = b1n;
@@ -675,13 +691,13 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // bias tile consumed: stage the next chunk's
             if (n < c_hi) stage_bias(n + 1);
           }
-          uint32_t dcw[2] = {0u, 0u};                 // keep bits of the chunk's 32 rows for this lane's two key columns
+          uint32_t dcw[NGK] = {};                       // keep bits of the chunk's 32 rows for this lane's two key columns
           if (DROP) {
-            const ACCT_LDS uint32_t* dc = (const ACCT_LDS uint32_t*)(qbuf + 2 * TILEB + STATB) + 2 * (pair * 64 + l32) + c;
+            const ACCT_LDS uint32_t* dc = (const ACCT_LDS uint32_t*)(qbuf + 2 * TILEB + STATB) + 2 * (pair * WK + l32) + c;
 #pragma unroll
-            for (int gk = 0; gk < 2; gk++) dcw[gk] = dc[64 * gk] >> (4 * g);
+            for (int gk = 0; gk < NGK; gk++) dcw[gk] = dc[64 * gk] >> (4 * g);
           }
-          V8 bfr[2][2];                               // B fragments of the second product: P (V role) or dS (K role)
+          V8 bfr[NGK][2];                              // B fragments of the second product: P (V role) or dS (K role)
           if (!krole) {
             if (edge) {
               // Side inputs and range limits are folded into the raw scores in place, in three short
@@ -692,7 +708,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
                 const int qlast = a.Sq - 1 - qc0;               // last valid row, relative to the chunk
                 const T* brow0 = alibip + (int64_t)qc0 * a.al_sq;
 #pragma unroll
-                for (int gk = 0; gk < 2; gk++) {
+                for (int gk = 0; gk < NGK; gk++) {
                   const int kv_c = min(wk0 + 32 * gk + l32, a.Sk - 1);
 #pragma unroll
                   for (int r = 0; r < 16; r++) {
@@ -709,7 +725,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
                                          : a.colbits + ((qc0 >> 5) & 3);
                 const uint32_t addbits = __float_as_uint(a.mask_add_raw);
 #pragma unroll
-                for (int gk = 0; gk < 2; gk++) {
+                for (int gk = 0; gk < NGK; gk++) {
                   const int kv_c = min(wk0 + 32 * gk + l32, a.Sk - 1);
                   const uint32_t w = cb[(a.mask_kind == kMaskDense ? kv_c : (kv_c & 127)) * 4] >> (4 * g);
 #pragma unroll
@@ -722,7 +738,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
               }
               if (limits)
 #pragma unroll
-              for (int gk = 0; gk < 2; gk++) {
+              for (int gk = 0; gk < NGK; gk++) {
                 const int kv = wk0 + 32 * gk + l32;
                 int lo = diag ? kv - qc0 - 4 * g : -64;         // chunk rows below it come before the key
                 int hi = a.Sq - 1 - qc0 - 4 * g;                // last query row that exists
@@ -735,7 +751,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
               }
             }
 #pragma unroll
-            for (int gk = 0; gk < 2; gk++) {
+            for (int gk = 0; gk < NGK; gk++) {
               const int kv_c = min(wk0 + 32 * gk + l32, a.Sk - 1);
 #pragma unroll
               for (int hh = 0; hh < 2; hh++) {
@@ -758,7 +774,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
             }
           } else {
 #pragma unroll
-            for (int gk = 0; gk < 2; gk++) {
+            for (int gk = 0; gk < NGK; gk++) {
               const int kv_c = min(wk0 + 32 * gk + l32, a.Sk - 1);
 #pragma unroll
               for (int hh = 0; hh < 2; hh++) {
@@ -799,7 +815,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
               const int db = i % C::DB, hh = i / C::DB;
               __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-              for (int gk = 0; gk < 2; gk++) acc[gk][db] = E::mfma(tr[i % BRING], bfr[gk][hh], acc[gk][db]);
+              for (int gk = 0; gk < NGK; gk++) acc[gk][db] = E::mfma(tr[i % BRING], bfr[gk][hh], acc[gk][db]);
               __builtin_amdgcn_sched_barrier(0);
               if (i + BRING < NT) tr[i % BRING] = tread(i + BRING);
             }
@@ -820,7 +836,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   constexpr int OPITCH = C::DB * 64 + 16;
   ACCT_LDS char* obuf = smem + wave * (32 * OPITCH);
 #pragma unroll
-  for (int gk = 0; gk < 2; gk++) {
+  for (int gk = 0; gk < NGK; gk++) {
 #pragma unroll
     for (int db = 0; db < C::DB; db++)
 #pragma unroll
@@ -852,7 +868,7 @@ template <typename T, int D, bool BIAS, bool DROP>
 static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
   hipError_t e = hipSuccess;
   if (stages & kStageDq) {
-    constexpr int QG = 1, NW = 8;
+    constexpr int QG = 1, NW = D > 128 ? 4 : 8;          // (wide head dims: one wave per SIMD has the registers)
     constexpr int BM = 32 * QG * NW;
     using CS = SwzCfg<D>;
     constexpr size_t tiles = 4 * 64 * (size_t)CS::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0) + (size_t)NW * 2 * DropRowStage<DROP, QG, 2>::BYTES, stage = (size_t)NW * 32 * (CS::DB * 64 + 16);
@@ -868,14 +884,15 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
   }
   if (stages & kStageDkDv) {
     using CS = SwzCfg<D>;
+    constexpr int NGK = dkdv_groups<D>();
     constexpr size_t stageb = 2 * 64 * (size_t)CS::PITCH + 512 + (DROP ? 2048 : 0);
-    constexpr size_t loopb = 2 * stageb + 8 * 4096 + 8 * (size_t)dkdv_park<D, BIAS, true>() * 1024 + (BIAS ? 4 * 4096 : 0),
+    constexpr size_t loopb = 2 * stageb + 8 * 2048 * NGK + 8 * (size_t)dkdv_park<D, BIAS, true>() * 1024 + (BIAS ? 4 * 4096 : 0),
                      epib = (size_t)8 * 32 * (CS::DB * 64 + 16);
     static_assert(loopb <= 160 * 1024 && epib <= 160 * 1024, "the workgroup's LDS must fit the CU's 160 KB");
     const size_t smem2 = loopb > epib ? loopb : epib;
-    a.n_tiles = (a.Sk + 255) / 256;
+    a.n_tiles = (a.Sk + 128 * NGK - 1) / (128 * NGK);
     const bool mask_t = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;
-    auto kern = mask_t ? fa_bwd_dkdv_kernel<T, D, BIAS, DROP, true> : fa_bwd_dkdv_kernel<T, D, BIAS, DROP, BIAS || DROP>;
+    auto kern = mask_t ? fa_bwd_dkdv_kernel<T, D, BIAS, DROP, true, NGK> : fa_bwd_dkdv_kernel<T, D, BIAS, DROP, BIAS || DROP, NGK>;
     e = allow_dynamic_lds((const void*)kern, smem2);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)((long long)a.n_tiles * a.B * a.N)), dim3(512), smem2, st, a);
@@ -884,15 +901,17 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
   return e;
 }
 
-template <typename T, int D>
+// SIDE = false: head dims 40 and 160, built without the bias and dropout variants
+template <typename T, int D, bool SIDE = true>
 static hipError_t launch_bwd_d(const FaArgs& a, int stages, hipStream_t st) {
   const bool bias = a.alibi != nullptr, drop = a.droprow != nullptr || a.dropcol != nullptr;
 #ifndef ACCT_DEV_BUILD
+  if constexpr (SIDE) {
   if (bias) return drop ? launch_bwd_t<T, D, true, true>(a, stages, st) : launch_bwd_t<T, D, true, false>(a, stages, st);
   if (drop) return launch_bwd_t<T, D, false, true>(a, stages, st);
-#else
-  if (bias || drop) return hipErrorNotSupported;       // development build: plain variants only
+  }
 #endif
+  if (bias || drop) return hipErrorNotSupported;       // (development build, head dims 40 / 160: plain variants only)
   return launch_bwd_t<T, D, false, false>(a, stages, st);
 }
 
@@ -912,10 +931,14 @@ hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t
     if (D == 128) return launch_bwd_d<f16, 128>(a, stages, st);
     if (D == 64) return launch_bwd_d<f16, 64>(a, stages, st);
     if (D == 80) return launch_bwd_d<f16, 80>(a, stages, st);
+    if (D == 40) return launch_bwd_d<f16, 40, false>(a, stages, st);
+    if (D == 160) return launch_bwd_d<f16, 160, false>(a, stages, st);
   } else {
     if (D == 128) return launch_bwd_d<bf16, 128>(a, stages, st);
     if (D == 64) return launch_bwd_d<bf16, 64>(a, stages, st);
     if (D == 80) return launch_bwd_d<bf16, 80>(a, stages, st);
+    if (D == 40) return launch_bwd_d<bf16, 40, false>(a, stages, st);
+    if (D == 160) return launch_bwd_d<bf16, 160, false>(a, stages, st);
   }
   return hipErrorInvalidValue;
 #endif

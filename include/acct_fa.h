@@ -37,7 +37,7 @@ extern "C" {
 #define ACCT_E_NULLPTR  (-1)   /* a required pointer is NULL */
 #define ACCT_E_SHAPE    (-2)   /* non-positive or inconsistent extent / stride */
 #define ACCT_E_DTYPE    (-3)   /* dtype is neither ACCT_F16 nor ACCT_BF16 */
-#define ACCT_E_HEADDIM  (-4)   /* D unsupported (64, 80, 128: forward and backward; 40, 160: forward only) */
+#define ACCT_E_HEADDIM  (-4)   /* D unsupported (built: 40, 64, 80, 128, 160; 40 and 160 without bias and dropout) */
 #define ACCT_E_ARCH     (-5)   /* current device is not gfx950 */
 #define ACCT_E_LAUNCH   (-6)   /* HIP reported a launch error */
 #define ACCT_E_WORKSPACE (-7)  /* workspace missing or too small */
@@ -179,8 +179,8 @@ int acct_fa_bwd_static(const acct_fa_params* p, const void* O, const void* dO, c
  * batch*heads 1..64, heads 1..4096, sequence lengths 1..8192 with k's equal to v's, D one of 40, 64, 80, 160
  * (a 3-D input is also held to the reference's 1..64 rule for its last dimension, :104-112).  Writes q's
  * extents to y_dims (may be NULL) and returns ACCT_OK, else an error code; no device is touched.
- * The operator itself is acct_fa_fwd with scale = 1, mask_kind = NONE (head dims 40 and 160 are built for
- * the forward only, without bias and dropout). */
+ * The operator itself is acct_fa_fwd with scale = 1, mask_kind = NONE (head dims 40 and 160 are built
+ * without the bias and dropout variants). */
 int acct_fa_infer_shape(const int64_t* q_dims, int q_rank, const int64_t* k_dims, int k_rank,
                         const int64_t* v_dims, int v_rank, int64_t* y_dims);
 

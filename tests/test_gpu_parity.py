@@ -592,25 +592,42 @@ def test_inference_operator_rejects_what_the_reference_rejects():
 
 
 @pytest.mark.parametrize("D, dtype", [(40, torch.float16), (160, torch.float16), (160, torch.bfloat16), (40, torch.bfloat16)])
-def test_forward_only_head_dims_with_masks(D, dtype):
-    # the forward kernel of the two extra head dims through the C ABI: scale, causal mask with block skip,
-    # dense mask, ragged lengths -- against the fp64 operator spec
+def test_extra_head_dims_with_masks(D, dtype):
+    # head dims 40 and 160 (the reference's wukong strategy and inference operator) through the C ABI, forward and
+    # backward: scale, causal mask with block skip, dense mask, ragged lengths -- against the fp64 operator spec
     B, N, Sq, Sk = 2, 2, 333, 460
     tol = dict(atol=ATOL_BF16, rtol=RTOL_BF16) if dtype == torch.bfloat16 else {}
-    q, k, v = (_gen(s, 810 + i, dtype) for i, s in enumerate([(B, N, Sq, D), (B, N, Sk, D), (B, N, Sk, D)]))
+    q, k, v, dO = (_gen(s, 810 + i, dtype) for i, s in enumerate([(B, N, Sq, D), (B, N, Sk, D), (B, N, Sk, D), (B, N, Sq, D)]))
     rng = np.random.default_rng(9)
     mask = (rng.random((B, Sq, Sk)) < 0.3).astype(np.uint8)
     mask[:, :, 0] = 0
-    _check_all(q, k, v, None, dict(scale=D ** -0.5, attn_mask=mask),
-               _run(q, k, v, scale=D ** -0.5, mask_kind=_capi.MASK_DENSE_U8, attn_mask=mask), **tol)
+    _check_all(q, k, v, dO, dict(scale=D ** -0.5, attn_mask=mask),
+               _run(q, k, v, dO, scale=D ** -0.5, mask_kind=_capi.MASK_DENSE_U8, attn_mask=mask), **tol)
     S = 384
-    q, k, v = (_gen((B, N, S, D), 820 + i, dtype) for i in range(3))
+    q, k, v, dO = (_gen((B, N, S, D), 820 + i, dtype) for i in range(4))
     tri = np.triu(np.ones((1, S, S), dtype=np.uint8), 1)
-    _check_all(q, k, v, None, dict(scale=D ** -0.5, attn_mask=tri),
-               _run(q, k, v, scale=D ** -0.5, mask_kind=_capi.MASK_CAUSAL, nxt=0), **tol)
+    _check_all(q, k, v, dO, dict(scale=D ** -0.5, attn_mask=tri),
+               _run(q, k, v, dO, scale=D ** -0.5, mask_kind=_capi.MASK_CAUSAL, nxt=0), **tol)
+    # bias and dropout are not built for these head dims
     with pytest.raises(_capi.AcctError) as e:
-        _run(q, k, v, _gen((B, N, S, D), 830, dtype), scale=1.0)
+        _run(q, k, v, dO, scale=1.0, keep_prob=0.9, drop_seed=3)
     assert e.value.code == -4
+
+
+@pytest.mark.parametrize("D, Sq, Sk", [(40, 4096, 4096), (40, 4096, 77), (80, 1024, 77), (160, 256, 256), (160, 64, 77), (160, 1024, 1024)])
+def test_wukong_training_shapes(D, Sq, Sk):
+    # the sequence lengths and head dims the reference's wukong tiling strategy is written for (self attention at
+    # 4096 / 1024 / 256 / 64 query rows, cross attention onto 77 keys; tiling_strategy/wukong_tiling.py:27-66),
+    # through the operator with tiling_stgy_name='wukong', forward and backward, no mask
+    B, N = 1, 2
+    q, dO = _gen((B, N, Sq, D), 840), _gen((B, N, Sq, D), 843)
+    k, v = _gen((B, N, Sk, D), 841), _gen((B, N, Sk, D), 842)
+    fa = get_flash_attention(tiling_stgy_name="wukong", scale=D ** -0.5)
+    qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    o, lse = fa(qd, kd, vd)
+    o.backward(dO.to(DEV))
+    torch.cuda.synchronize()
+    _check_all(q, k, v, dO, dict(scale=D ** -0.5), (o, lse, (qd.grad, kd.grad, vd.grad)))
 
 
 def test_layer_dropout_follows_torch_seed_and_call_count():
@@ -768,6 +785,49 @@ def test_operator_takes_reference_form_masks_without_conversion():
     o.backward(dO.to(DEV))
     torch.cuda.synchronize()
     _check_all(q, k, v, dO, dict(scale=D ** -0.5, attn_mask=m8, drop_mask=d8, keep_prob=0.75), (o, lse, (qd.grad, kd.grad, vd.grad)))
+
+
+# ---- the MindSpore AOT custom-op adapter over the C ABI ------------------------------------------------
+def test_mindspore_aot_adapter_forward_and_backward():
+    # libacct_fa_ms.so driven the way MindSpore drives an AOT custom op: (nparam, params, ndims, shapes, dtypes,
+    # stream, extra), operands in the reference's order (flash_attention_impl.py:113-114,150-153), masks in the
+    # reference's fp16 forms, absent optional inputs as NULL
+    from test_host_api import _ms_lib, ms_call_args
+    lib = _ms_lib()
+    B, N, S, D = 2, 2, 256, 128
+    q, k, v, dO = (_gen((B, N, S, D), s) for s in (190, 191, 192, 193))
+    m8 = np.triu(np.ones((S, S), np.uint8), 1)[None].repeat(B, 0); m8[1, :, 200:] = 1
+    d8 = (np.random.default_rng(194).random((B, N, S, S)) < 0.8).astype(np.uint8)
+    keep = 0.8
+    dev = lambda t: t.to(DEV)
+    qd, kd, vd, dod = dev(q), dev(k), dev(v), dev(dO)
+    mf, df = dev(torch.from_numpy(m8).half()), dev((torch.from_numpy(d8).float() / keep).half())
+    o, lse = torch.empty_like(qd), torch.empty(B, N, S, dtype=torch.float32, device=DEV)
+    attrs = (ctypes.c_int32 * 2)(65536, 65536)
+
+    class Attrs(ctypes.Structure):
+        _fields_ = [("prev_block_num", ctypes.c_int32), ("next_block_num", ctypes.c_int32), ("scale", ctypes.c_float), ("keep_prob", ctypes.c_float)]
+    at = Attrs(65536, 65536, D ** -0.5, keep)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sh, f16 = (B, N, S, D), "float16"
+    plib = _capi.load()
+    p = _capi.make_params(qd, kd, vd, scale=D ** -0.5, keep_prob=keep, mask_kind=_capi.MASK_DENSE_F16, attn_mask=mf, drop_mask=df)
+    ws = torch.empty(max(plib.acct_fa_fwd_workspace_bytes(ctypes.byref(p)), 256), dtype=torch.uint8, device=DEV)
+    ops = [(qd.data_ptr(), sh, f16), (kd.data_ptr(), sh, f16), (vd.data_ptr(), sh, f16), (mf.data_ptr(), (B, S, S), f16),
+           (df.data_ptr(), (B, N, S, S), f16), (None, (), f16),
+           (o.data_ptr(), sh, f16), (lse.data_ptr(), (B, N, S), "float32"), (ws.data_ptr(), (ws.numel(),), "uint8")]
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(ops)
+    assert lib.FlashAttentionFwd(n, params, ndims, shapes, dtypes, st, ctypes.addressof(at)) == 0, plib.acct_last_error().decode()
+    dq, dk, dv = (torch.empty_like(t) for t in (qd, kd, vd))
+    # no workspace output declared: the adapter takes the entry point that needs none
+    ops = [(qd.data_ptr(), sh, f16), (kd.data_ptr(), sh, f16), (vd.data_ptr(), sh, f16), (o.data_ptr(), sh, f16),
+           (dod.data_ptr(), sh, f16), (lse.data_ptr(), (B, N, S), "float32"), (mf.data_ptr(), (B, S, S), f16),
+           (df.data_ptr(), (B, N, S, S), f16), (None, (), f16),
+           (dq.data_ptr(), sh, f16), (dk.data_ptr(), sh, f16), (dv.data_ptr(), sh, f16)]
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(ops)
+    assert lib.FlashAttentionGrad(n, params, ndims, shapes, dtypes, st, ctypes.addressof(at)) == 0, plib.acct_last_error().decode()
+    torch.cuda.synchronize()
+    _check_all(q, k, v, dO, dict(scale=D ** -0.5, attn_mask=m8, drop_mask=d8, keep_prob=keep), (o, lse, (dq, dk, dv)))
 
 
 # ---- the reference's CPU-sized configuration through the HIP path ------------------------------------

@@ -126,7 +126,7 @@ def test_infer_shape_function():
     assert lib.acct_fa_infer_shape(None, 4, None, 4, None, 4, None) == -1
 
 
-def test_inference_head_dims_are_forward_only():
+def test_extra_head_dims_take_forward_and_backward_without_bias_and_dropout():
     lib = _capi.load()
     buf = (ctypes.c_char * 64)()
     a = ctypes.addressof(buf)
@@ -135,7 +135,8 @@ def test_inference_head_dims_are_forward_only():
         p = _capi.make_params(q, q.clone(), q.clone(), scale=1.0)
         # the forward accepts the head dim (the call gets past validation to the NULL output check: nothing is launched)
         assert lib.acct_fa_fwd(ctypes.byref(p), None, None, None, 0, None) == -1
-        assert lib.acct_fa_bwd(ctypes.byref(p), *([a] * 6), None, 0, None) == -4
+        # so does the backward (it gets past validation to the workspace check)
+        assert lib.acct_fa_bwd(ctypes.byref(p), *([a] * 6), None, 0, None) == -7
         p2 = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, keep_prob=0.9, drop_seed=1)
         assert lib.acct_fa_fwd(ctypes.byref(p2), None, None, None, 0, None) == -4
 
@@ -282,3 +283,44 @@ def test_oracle_reproduces_golden(name):
     dQ, dK, dV = orc.unfused_bwd(c["q"], c["k"], c["v"], c["dO"], **kw)
     for got, want in ((O, c["O"]), (L, c["L"]), (dQ, c["dQ"]), (dK, c["dK"]), (dV, c["dV"])):
         assert np.allclose(got, want, rtol=1e-6, atol=1e-6)
+
+
+# ---- the MindSpore AOT custom-op adapter (libacct_fa_ms.so) ---------------------------------------------
+def _ms_lib():
+    lib = ctypes.CDLL(os.path.join(ROOT, "acctransformer_amd", "libacct_fa_ms.so"))
+    for name in ("FlashAttentionFwd", "FlashAttentionGrad"):
+        fn = getattr(lib, name)
+        fn.restype = ctypes.c_int
+        fn.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_int),
+                       ctypes.POINTER(ctypes.POINTER(ctypes.c_int64)), ctypes.POINTER(ctypes.c_char_p), ctypes.c_void_p, ctypes.c_void_p]
+    return lib
+
+
+def ms_call_args(operands):
+    """(nparam, params, ndims, shapes, dtypes) of MindSpore's AOT convention from a list of (pointer or None, shape, dtype name)."""
+    n = len(operands)
+    params = (ctypes.c_void_p * n)(*[op[0] for op in operands])
+    ndims = (ctypes.c_int * n)(*[len(op[1]) for op in operands])
+    rows = [(ctypes.c_int64 * max(len(op[1]), 1))(*op[1]) for op in operands]
+    shapes = (ctypes.POINTER(ctypes.c_int64) * n)(*[ctypes.cast(r, ctypes.POINTER(ctypes.c_int64)) for r in rows])
+    dtypes = (ctypes.c_char_p * n)(*[op[2].encode() for op in operands])
+    return n, params, ndims, shapes, dtypes, rows
+
+
+def test_mindspore_adapter_loads_and_validates_without_a_device():
+    lib = _ms_lib()
+    buf = (ctypes.c_char * 64)()
+    a = ctypes.addressof(buf)
+    sh = (1, 2, 128, 128)
+    good = [(a, sh, "float16")] * 3 + [(None, (), "float16")] * 3 + [(a, sh, "float16"), (a, sh[:3], "float32")]
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(good)
+    assert lib.FlashAttentionFwd(3, params, ndims, shapes, dtypes, None, None) == -1          # too few operands
+    bad = list(good); bad[1] = (a, sh, "float32")
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(bad)
+    assert lib.FlashAttentionFwd(n, params, ndims, shapes, dtypes, None, None) == -3          # q, k, v dtypes differ
+    bad = list(good); bad[3] = (a, (1, 100, 128), "float16")
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(bad)
+    assert lib.FlashAttentionFwd(n, params, ndims, shapes, dtypes, None, None) == -2          # mask shape
+    bad = list(good); bad[3] = (a, (1, 128, 128), "int32")
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(bad)
+    assert lib.FlashAttentionFwd(n, params, ndims, shapes, dtypes, None, None) == -3          # mask dtype
