@@ -13,6 +13,22 @@ pair and the library draws the keep decisions itself (Philox4x32-10), the same
 in forward and backward, and applies the 1/keep_prob factor inside the kernel.
 The seed follows torch's global seed, so `torch.manual_seed` makes a run
 repeatable.
+
+Differences from the reference Cell that a caller can see:
+  * Dropout is applied in training mode only (`module.train()`), the torch
+    convention; the reference applies it whenever `dropout_rate > 0`
+    (`:198-203`).  Call `.train()` to get the reference's behaviour.
+  * The keep probability actually used is `round(256 * keep_prob) / 256`
+    (the keep decision compares one random byte with a threshold), e.g.
+    0.9 -> 230/256 = 0.8984; kept probabilities are scaled by the
+    reciprocal of that value, so the expectation is exact.
+  * The dropout stream of a call is (seed, offset) = (torch's seed mixed
+    with a per-layer id, a per-layer call counter).  The counter is Python
+    state: a forward that is re-run (activation checkpointing) would draw a
+    new mask.  Pass `dropout_state=(seed, offset)` to `forward` to fix the
+    stream of a call explicitly; the same pair reproduces the same mask.
+  * Head dims built: 40, 64, 80, 128, 160 (the reference admits any
+    multiple of 16 up to 256); others raise when the op is called.
 """
 from __future__ import annotations
 
@@ -84,7 +100,7 @@ class FlashAttention(torch.nn.Module):
         self.dp, self.mp = in_strategy[0][0], in_strategy[0][1]
         return self
 
-    def forward(self, q, k, v, attn_mask=None, alibi_mask=None):
+    def forward(self, q, k, v, attn_mask=None, alibi_mask=None, dropout_state=None):
         bsz, head_num, seq_len, head_dim = q.shape
         _, k_head_num, _, _ = k.shape
         _, v_head_num, _, _ = v.shape
@@ -93,9 +109,12 @@ class FlashAttention(torch.nn.Module):
                 "the head_num of query, key and value must be the same, "
                 "If different head_num are used, users need to change themselves to be same by tile.")
         if self.enable_dropout and self.training:
-            seed = (torch.initial_seed() ^ (self._layer_id * 0x9E3779B97F4A7C15)) & 0xFFFFFFFFFFFFFFFF
-            drop_mask = (seed, self._calls & 0xFFFFFFFF)
-            self._calls += 1
+            if dropout_state is not None:             # the caller fixes the stream (e.g. a checkpointed forward that is re-run)
+                drop_mask = (int(dropout_state[0]) & 0xFFFFFFFFFFFFFFFF, int(dropout_state[1]) & 0xFFFFFFFF)
+            else:
+                seed = (torch.initial_seed() ^ (self._layer_id * 0x9E3779B97F4A7C15)) & 0xFFFFFFFFFFFFFFFF
+                drop_mask = (seed, self._calls & 0xFFFFFFFF)
+                self._calls += 1
         else:
             drop_mask = None
         o, _ = self.flash_attention(q, k, v, attn_mask, drop_mask, alibi_mask)

@@ -13,6 +13,11 @@ block_size) of the reference's row-block prefixes, the kernel never visits a
 blocks that mix masked and unmasked entries.  When block_size is not a
 multiple of 128 (the kernel's block granularity) the row blocks are launched
 one by one on views of q, k, v, as the reference slices them.
+
+Dropout follows the FlashAttention layer here: training mode only, keep
+probability rounded to a multiple of 1/256, one (seed, offset) stream per call
+from torch's seed and a per-layer call counter; `dropout_state=(seed, offset)`
+fixes the stream of a call (a re-run forward then draws the same mask).
 """
 from __future__ import annotations
 
@@ -52,14 +57,17 @@ class TriangleAttention(torch.nn.Module):
                                        row_block_prefix=block_size if self._fused else 0)
         self._calls = 0                               # one fresh dropout mask per training call
 
-    def forward(self, query, key, value, attention_mask):
+    def forward(self, query, key, value, attention_mask, dropout_state=None):
         bsz, head_num, seq_len, _ = query.shape
         # dropout: no mask tensor, the library draws the keep decisions from a (seed, offset) pair
         dropping = self.enable_dropout and self.training
-        seed = (torch.initial_seed() ^ 0x7F4A7C15F39CC060) & 0xFFFFFFFFFFFFFFFF
-        call = self._calls
-        if dropping:
-            self._calls += 1
+        if dropout_state is not None:
+            seed, call = int(dropout_state[0]) & 0xFFFFFFFFFFFFFFFF, int(dropout_state[1])
+        else:
+            seed = (torch.initial_seed() ^ 0x7F4A7C15F39CC060) & 0xFFFFFFFFFFFFFFFF
+            call = self._calls
+            if dropping:
+                self._calls += 1
         if self._fused:
             o, _ = self._op(query, key, value, attention_mask, (seed, call & 0xFFFFFFFF) if dropping else None, None)
             return o

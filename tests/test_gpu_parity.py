@@ -630,6 +630,22 @@ def test_wukong_training_shapes(D, Sq, Sk):
     _check_all(q, k, v, dO, dict(scale=D ** -0.5), (o, lse, (qd.grad, kd.grad, vd.grad)))
 
 
+def test_layer_dropout_state_can_be_fixed_by_the_caller():
+    # a forward that is run again (activation checkpointing) must draw the same mask: dropout_state fixes the stream
+    B, N, S, D = 1, 2, 256, 64
+    q, k, v = (_gen((B, N, S, D), s).to(DEV) for s in (860, 861, 862))
+    layer = FlashAttention(head_dim=D, dropout_rate=0.2).train()
+    a = layer(q, k, v, dropout_state=(99, 5))
+    b = layer(q, k, v, dropout_state=(99, 5))
+    c = layer(q, k, v, dropout_state=(99, 6))
+    d = layer(q, k, v)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b) and not torch.equal(a, c) and not torch.equal(a, d)
+    tri = TriangleAttention(block_size=128, dropout_rate=0.2).train()
+    m = torch.triu(torch.ones(B, S, S, dtype=torch.uint8, device=DEV), 1)
+    assert torch.equal(tri(q, k, v, m, dropout_state=(7, 1)), tri(q, k, v, m, dropout_state=(7, 1)))
+
+
 def test_layer_dropout_follows_torch_seed_and_call_count():
     # the layers hand the op (seed, offset): torch's seed makes a run repeatable, every training call
     # draws a fresh mask, and the gradients see the mask of their own forward
