@@ -91,10 +91,11 @@ int validate(const acct_fa_params* p, bool backward) {
     return fail(ACCT_E_SHAPE, "extents must be positive: B=%d N=%d Sq=%d Sk=%d D=%d", p->B, p->N, p->Sq, p->Sk, p->D);
   if (p->D > 256) return fail(ACCT_E_HEADDIM, "head_dim too large, reduce head_dim and try again. (D=%d > 256)", p->D);
   const bool d_train = p->D == 64 || p->D == 80 || p->D == 128;
-  const bool d_infer = p->D == 40 || p->D == 160;           // no bias / dropout: the inference operator's and the wukong strategy's other head dims
+  const bool d_infer = p->D == 40 || p->D == 160 || p->D == 256;   // no bias / dropout: the inference operator's and the wukong strategy's
+                                                                   // other head dims, and the layer's maximum
   (void)backward;
   if (!d_train && !d_infer)
-    return fail(ACCT_E_HEADDIM, "head_dim %d not built; supported: 40, 64, 80, 128, 160", p->D);
+    return fail(ACCT_E_HEADDIM, "head_dim %d not built; supported: 40, 64, 80, 128, 160, 256", p->D);
   if (d_infer && (p->alibi || p->drop_mask || (p->drop_philox && p->keep_prob < 1.f)))
     return fail(ACCT_E_HEADDIM, "head_dim %d is built without the bias and dropout variants", p->D);
   if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return fail(ACCT_E_PARAM, "scale must be positive and finite, got %g", (double)p->scale);

@@ -38,7 +38,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   constexpr int BM = 32 * QG * NW;
   constexpr int TILEB = 64 * C::PITCH;
   constexpr int FRING = 4, TRING = 3;                     // fragment reads in flight ahead of their MFMA (row-major / transposed)
-  constexpr bool RINGS = !(BIAS || DROP) && D <= 128;     // (the side-input variants and the wide head dims have no registers for the rings)   // fragment reads in flight ahead of their MFMA (row-major / transposed)
+  constexpr bool RINGS = !(BIAS || DROP);                 // (the side-input variants have no registers for the rings)   // fragment reads in flight ahead of their MFMA (row-major / transposed)
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 buffers][K tile | V tile]; reused by the epilogue
 
@@ -115,9 +115,13 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   }
 
   // per-lane LDS offsets (tile-invariant)
-  int koff[C::KS];
+  // row-major fragment of k-step t: row l32, chunk 2t + g.  Chunk c + 8 of a row sits in slot (c ^ swz) ^ 8, so the
+  // offsets of the upper parts of a wide head dim are one XOR away from the first four.
+  constexpr int NKOFF = (C::CH >= 16 && C::KS > 8) ? 4 : C::KS;
+  int koff_[NKOFF];
 #pragma unroll
-  for (int t = 0; t < C::KS; t++) koff[t] = l32 * C::PITCH + swz_off(2 * t + g, C::swz(l32));
+  for (int t = 0; t < NKOFF; t++) koff_[t] = l32 * C::PITCH + swz_off(2 * t + g, C::swz(l32));
+  auto koff = [&](int t) { return t < NKOFF ? koff_[t] : (koff_[t & 3] ^ ((t >> 2) * 128)); };
   const int trow = 4 * g + ((lane & 15) >> 2);
   const int tchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
   int toff[C::DB];
@@ -225,7 +229,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
             // flight ahead of the MFMA that consumes the oldest); S and dP MFMAs alternate.  The scheduling
             // barriers keep the compiler from folding the ring back into read-wait-MFMA.
             constexpr int NF = 2 * C::KS;
-            auto faddr = [&](int i) { return ((i & 1) ? vbuf : kbuf) + koff[i >> 1] + c * 32 * C::PITCH; };
+            auto faddr = [&](int i) { return ((i & 1) ? vbuf : kbuf) + koff(i >> 1) + c * 32 * C::PITCH; };
             V8 ring[FRING];
 #pragma unroll
             for (int i = 0; i < FRING; i++) ring[i] = lds_read_frag<T>(faddr(i));
@@ -244,9 +248,9 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
           } else {
             V8 kf[C::KS], vf[C::KS];
 #pragma unroll
-            for (int t = 0; t < C::KS; t++) kf[t] = lds_read_frag<T>(kbuf + koff[t] + c * 32 * C::PITCH);
+            for (int t = 0; t < C::KS; t++) kf[t] = lds_read_frag<T>(kbuf + koff(t) + c * 32 * C::PITCH);
 #pragma unroll
-            for (int t = 0; t < C::KS; t++) vf[t] = lds_read_frag<T>(vbuf + koff[t] + c * 32 * C::PITCH);
+            for (int t = 0; t < C::KS; t++) vf[t] = lds_read_frag<T>(vbuf + koff(t) + c * 32 * C::PITCH);
 #pragma unroll
             for (int t = 0; t < C::KS; t++)
 #pragma unroll
@@ -933,12 +937,14 @@ hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t
     if (D == 80) return launch_bwd_d<f16, 80>(a, stages, st);
     if (D == 40) return launch_bwd_d<f16, 40, false>(a, stages, st);
     if (D == 160) return launch_bwd_d<f16, 160, false>(a, stages, st);
+    if (D == 256) return launch_bwd_d<f16, 256, false>(a, stages, st);
   } else {
     if (D == 128) return launch_bwd_d<bf16, 128>(a, stages, st);
     if (D == 64) return launch_bwd_d<bf16, 64>(a, stages, st);
     if (D == 80) return launch_bwd_d<bf16, 80>(a, stages, st);
     if (D == 40) return launch_bwd_d<bf16, 40, false>(a, stages, st);
     if (D == 160) return launch_bwd_d<bf16, 160, false>(a, stages, st);
+    if (D == 256) return launch_bwd_d<bf16, 256, false>(a, stages, st);
   }
   return hipErrorInvalidValue;
 #endif

@@ -481,12 +481,14 @@ hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st)
     if (D == 80) return launch_fwd_d<f16, 80>(a, qg, st);
     if (D == 40) return launch_fwd_plain<f16, 40>(a, qg, st);
     if (D == 160) return launch_fwd_plain<f16, 160>(a, qg, st);
+    if (D == 256) return launch_fwd_q<f16, 256, 1, 4, false>(a, st);     // one wave per SIMD: 128 accumulator registers
   } else {
     if (D == 128) return launch_fwd_d<bf16, 128>(a, qg, st);
     if (D == 64) return launch_fwd_d<bf16, 64>(a, qg, st);
     if (D == 80) return launch_fwd_d<bf16, 80>(a, qg, st);
     if (D == 40) return launch_fwd_plain<bf16, 40>(a, qg, st);
     if (D == 160) return launch_fwd_plain<bf16, 160>(a, qg, st);
+    if (D == 256) return launch_fwd_q<bf16, 256, 1, 4, false>(a, st);
   }
   return hipErrorInvalidValue;
 #endif

@@ -27,7 +27,7 @@ Differences from the reference Cell that a caller can see:
     state: a forward that is re-run (activation checkpointing) would draw a
     new mask.  Pass `dropout_state=(seed, offset)` to `forward` to fix the
     stream of a call explicitly; the same pair reproduces the same mask.
-  * Head dims built: 40, 64, 80, 128, 160 (the reference admits any
+  * Head dims built: 40, 64, 80, 128, 160, 256 (the reference admits any
     multiple of 16 up to 256); others raise when the op is called.
 """
 from __future__ import annotations

@@ -268,6 +268,11 @@ def main():
         fl5 = 14.0 * B5 * N5 * S5 * S5 * D * f5
         pp = _capi.make_params(q5, k5, v5, scale=scale, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m5, drop_mask=dr5)
         run_config("padded_dropout_B16_N16_S1024_mask_tensor", pp, q5, k5, v5, d5, fl5, 2 * (m5.numel() + dr5.numel()))
+        # the same masks in the reference's own form: fp16 attn_mask (1 = masked) and fp16 {0, 1/keep_prob} dropout mask
+        m5f, dr5f = m5.half(), (dr5.half() / 0.9).half()
+        pp = _capi.make_params(q5, k5, v5, scale=scale, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_F16, attn_mask=m5f, drop_mask=dr5f)
+        run_config("padded_dropout_B16_N16_S1024_fp16_mask_tensors", pp, q5, k5, v5, d5, fl5, 2 * 2 * (m5.numel() + dr5.numel()))
+        del m5f, dr5f
         pp = _capi.make_params(q5, k5, v5, scale=scale, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m5, drop_seed=1234)
         run_config("padded_dropout_B16_N16_S1024_seed_pair", pp, q5, k5, v5, d5, fl5, 2 * m5.numel())
         other["padded_dropout_unmasked_fraction"] = round(f5, 4)

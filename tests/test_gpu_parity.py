@@ -591,9 +591,11 @@ def test_inference_operator_rejects_what_the_reference_rejects():
         flash_attention_tik(*(z(2, 2, 128, 64).to(torch.bfloat16) for _ in range(3)))
 
 
-@pytest.mark.parametrize("D, dtype", [(40, torch.float16), (160, torch.float16), (160, torch.bfloat16), (40, torch.bfloat16)])
+@pytest.mark.parametrize("D, dtype", [(40, torch.float16), (160, torch.float16), (160, torch.bfloat16), (40, torch.bfloat16),
+                                      (256, torch.float16), (256, torch.bfloat16)])
 def test_extra_head_dims_with_masks(D, dtype):
-    # head dims 40 and 160 (the reference's wukong strategy and inference operator) through the C ABI, forward and
+    # head dims 40, 160 (the reference's wukong strategy and inference operator) and 256 (the layer's limit,
+    # nn/layer/flash_attention.py:26,105-106) through the C ABI, forward and
     # backward: scale, causal mask with block skip, dense mask, ragged lengths -- against the fp64 operator spec
     B, N, Sq, Sk = 2, 2, 333, 460
     tol = dict(atol=ATOL_BF16, rtol=RTOL_BF16) if dtype == torch.bfloat16 else {}

@@ -96,6 +96,23 @@ def test_null_outputs_and_workspace_sizes():
     assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p2)) == 2 * (2 * 2 * 128 * 4) + 256 + 1 * 1 * 128 * 16
 
 
+def test_forward_rejects_misaligned_output_and_workspace():
+    # O is stored in 16-byte rows and the workspace regions are 256-byte aligned: a misaligned pointer is an error
+    # code, not a misaligned vector access (checked before any device is touched)
+    lib = _capi.load()
+    raw = (ctypes.c_char * 1024)()
+    base = (ctypes.addressof(raw) + 255) // 256 * 256
+    p = _params()
+    assert lib.acct_fa_fwd(ctypes.byref(p), base + 8, base, None, 0, None) == -2
+    m = torch.zeros(1, 128, 128, dtype=torch.uint8)
+    q = torch.zeros(1, 2, 128, 128, dtype=torch.float16)
+    p2 = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m)
+    need = lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p2))
+    assert need > 0
+    assert lib.acct_fa_fwd(ctypes.byref(p2), base, base, base + 64, need, None) == -7
+    assert "aligned" in lib.acct_last_error().decode()
+
+
 def test_infer_shape_function():
     # accept / reject cases of the inference operator's shape function
     # (infer/flash_attention/tik/op_proto/flash_attention_tik.cpp:20-193 of the reference)
@@ -130,7 +147,7 @@ def test_extra_head_dims_take_forward_and_backward_without_bias_and_dropout():
     lib = _capi.load()
     buf = (ctypes.c_char * 64)()
     a = ctypes.addressof(buf)
-    for D in (40, 160):
+    for D in (40, 160, 256):
         q = torch.zeros(1, 2, 128, D, dtype=torch.float16)
         p = _capi.make_params(q, q.clone(), q.clone(), scale=1.0)
         # the forward accepts the head dim (the call gets past validation to the NULL output check: nothing is launched)
