@@ -90,13 +90,11 @@ int validate(const acct_fa_params* p, bool backward) {
   if (p->B <= 0 || p->N <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->D <= 0)
     return fail(ACCT_E_SHAPE, "extents must be positive: B=%d N=%d Sq=%d Sk=%d D=%d", p->B, p->N, p->Sq, p->Sk, p->D);
   if (p->D > 256) return fail(ACCT_E_HEADDIM, "head_dim too large, reduce head_dim and try again. (D=%d > 256)", p->D);
-  const bool d_train = p->D == 64 || p->D == 80 || p->D == 128;
-  const bool d_infer = p->D == 40 || p->D == 160 || p->D == 256;   // no bias / dropout: the inference operator's and the wukong strategy's
-                                                                   // other head dims, and the layer's maximum
+  if (p->D % 8 != 0) return fail(ACCT_E_HEADDIM, "head_dim %d is not a multiple of 8", p->D);
   (void)backward;
-  if (!d_train && !d_infer)
-    return fail(ACCT_E_HEADDIM, "head_dim %d not built; supported: 40, 64, 80, 128, 160, 256", p->D);
-  if (d_infer && (p->alibi || p->drop_mask || (p->drop_philox && p->keep_prob < 1.f)))
+  // bias and dropout variants are built for the head-dim classes 64, 80 and 128
+  const bool no_side = p->D == 40 || p->D > 128;
+  if (no_side && (p->alibi || p->drop_mask || (p->drop_philox && p->keep_prob < 1.f)))
     return fail(ACCT_E_HEADDIM, "head_dim %d is built without the bias and dropout variants", p->D);
   if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return fail(ACCT_E_PARAM, "scale must be positive and finite, got %g", (double)p->scale);
   if (!(p->keep_prob > 0.f && p->keep_prob <= 1.f)) return fail(ACCT_E_PARAM, "keep_prob must be in (0, 1], got %g", (double)p->keep_prob);
@@ -146,6 +144,7 @@ acct::FaArgs make_args(const acct_fa_params* p) {
   a.drop_es = p->drop_mask_kind == ACCT_DROP_F16 ? 2 : 1;
   a.alibi = p->alibi;
   a.B = p->B; a.N = p->N; a.Sq = p->Sq; a.Sk = p->Sk;
+  a.hd = p->D;
   a.Tr = (p->Sq + 127) / 128; a.Tc = (p->Sk + 127) / 128;
   fill_strides(p->q_stride, p->N, p->Sq, p->D, &a.q_sb, &a.q_sh, &a.q_ss);
   fill_strides(p->k_stride, p->N, p->Sk, p->D, &a.k_sb, &a.k_sh, &a.k_ss);

@@ -90,9 +90,9 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
     float part = 0.f;
 #pragma unroll
     for (int t = 0; t < C::KS; t++) {
-      // D % 16 == 8: the upper half of the last k-step lies past the row; zeros there make the products
+      // k-steps (or the upper half of one) past the head dim: zeros there make the products
       // ignore whatever the K / V tiles hold in that slot
-      const bool inside = (D % 16 == 0) || 16 * t + 8 * g < D;
+      const bool inside = 16 * t + 8 * g < a.hd;
       V8 z;
 #pragma unroll
       for (int e = 0; e < 8; e++) z[e] = 0;
@@ -144,8 +144,9 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
   TileDma<T, D, 64, NW> kdma, vdma;
-  kdma.plan(a.k_ss);
-  vdma.plan(a.v_ss);
+  const int cpr = a.hd >> 3;                                // valid 16-byte chunks per row
+  kdma.plan(a.k_ss, cpr);
+  vdma.plan(a.v_ss, cpr);
   // bias tiles of this wave's rows are staged through a wave-private LDS region one tile ahead
   ACCT_LDS char* bias_lds = smem + 4 * TILEB + wave * (QG * 4096);
   const bool bias_staged = BIAS && (a.Sk & 7) == 0 && (((uintptr_t)a.alibi & 15) | ((a.al_sb | a.al_sh | a.al_sq) & 7)) == 0;
@@ -158,8 +159,8 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   using DropStage = DropRowStage<DROP, QG, 2>;
   ACCT_LDS char* drop_lds = smem + 4 * TILEB + (BIAS ? NW * QG * 4096 : 0) + wave * (2 * DropStage::BYTES);
   if (j_lo <= j_hi) {
-    tile_dma<T, D, 64, NW>(kp, a.k_ss, j_lo * 64, a.Sk, smem);
-    tile_dma<T, D, 64, NW>(vp, a.v_ss, j_lo * 64, a.Sk, smem + TILEB);
+    tile_dma<T, D, 64, NW>(kp, a.k_ss, j_lo * 64, a.Sk, smem, a.hd >> 3);
+    tile_dma<T, D, 64, NW>(vp, a.v_ss, j_lo * 64, a.Sk, smem + TILEB, a.hd >> 3);
     if (BIAS && bias_staged && wq0 < a.Sq) stage_bias(j_lo);
     DropStage::issue(a, bh, wq0, j_lo, lane, drop_lds);
     // A full wait the compiler can see: every load issued so far (Q, dO fragments included) is complete,
@@ -182,8 +183,8 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
           kdma.issue(kp, a.k_ss, (j + 1) * 64, nb);
           vdma.issue(vp, a.v_ss, (j + 1) * 64, nb + TILEB);
         } else {                                            // ragged last tile: clamped rows
-          tile_dma<T, D, 64, NW>(kp, a.k_ss, (j + 1) * 64, a.Sk, nb);
-          tile_dma<T, D, 64, NW>(vp, a.v_ss, (j + 1) * 64, a.Sk, nb + TILEB);
+          tile_dma<T, D, 64, NW>(kp, a.k_ss, (j + 1) * 64, a.Sk, nb, a.hd >> 3);
+          tile_dma<T, D, 64, NW>(vp, a.v_ss, (j + 1) * 64, a.Sk, nb + TILEB, a.hd >> 3);
         }
         DropStage::issue(a, bh, wq0, j + 1, lane, drop_lds + (buf ^ 1) * DropStage::BYTES);
       }
@@ -400,13 +401,14 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
         typename E::V4 ov = {t0[0], t0[1], t1[0], t1[1]};
         *reinterpret_cast<ACCT_LDS typename E::V4*>(obuf + l32 * OPITCH + (32 * db + 8 * r4 + 4 * g) * 2) = ov;
       }
-    constexpr int NCH = C::CPR;
+    const int nch = a.hd >> 3;                       // valid 16-byte chunks per row
+    const uint32_t nch_inv = recip16(nch);
 #pragma unroll
-    for (int i = 0; i < (32 * NCH + 63) / 64; i++) {
+    for (int i = 0; i < (32 * C::CPR + 63) / 64; i++) {
       const int idx = lane + 64 * i;
-      const int r = idx / NCH, ch = idx % NCH;
+      const int r = div_small(idx, nch_inv), ch = idx - r * nch;
       const int grow = wq0 + 32 * gq + r;
-      if (idx < 32 * NCH && grow < a.Sq) {
+      if (idx < 32 * nch && grow < a.Sq) {
         const u32x4 v = *reinterpret_cast<const ACCT_LDS u32x4*>(obuf + r * OPITCH + ch * 16);
         *reinterpret_cast<u32x4*>(dqp + (int64_t)grow * a.q_ss + ch * 8) = v;
       }
@@ -503,9 +505,9 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
       const int row = min(wk0 + 32 * gk + l32, a.Sk - 1);
 #pragma unroll
       for (int t = 0; t < C::KS; t++) {
-        // D % 16 == 8: the upper half of the last k-step lies past the row; zeros there make the products
+        // k-steps (or the upper half of one) past the head dim: zeros there make the products
         // ignore whatever the Q / dO tiles hold in that slot
-        const bool inside = (D % 16 == 0) || 16 * t + 8 * g < D;
+        const bool inside = 16 * t + 8 * g < a.hd;
         V8 v;
 #pragma unroll
         for (int e = 0; e < 8; e++) v[e] = 0;
@@ -536,11 +538,11 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   // (addresses are re-derived per call here: this kernel has no registers to spare for a TileDma plan)
   auto stage = [&](int i, ACCT_LDS char* sb) {
     if ((i + 1) * 64 <= a.Sq) {
-      TileDma<T, D, 64, NW>::issue_direct(qp, a.q_ss, i * 64, sb);
-      TileDma<T, D, 64, NW>::issue_direct(dop, a.o_ss, i * 64, sb + TILEB);
+      TileDma<T, D, 64, NW>::issue_direct(qp, a.q_ss, i * 64, sb, a.hd >> 3);
+      TileDma<T, D, 64, NW>::issue_direct(dop, a.o_ss, i * 64, sb + TILEB, a.hd >> 3);
     } else {                                         // ragged last tile: clamped rows
-      tile_dma<T, D, 64, NW>(qp, a.q_ss, i * 64, a.Sq, sb);
-      tile_dma<T, D, 64, NW>(dop, a.o_ss, i * 64, a.Sq, sb + TILEB);
+      tile_dma<T, D, 64, NW>(qp, a.q_ss, i * 64, a.Sq, sb, a.hd >> 3);
+      tile_dma<T, D, 64, NW>(dop, a.o_ss, i * 64, a.Sq, sb + TILEB, a.hd >> 3);
     }
     if (wave < 2) {                                  // (pointers rebuilt from the kernel arguments: nothing to keep live)
       const int r = min(i * 64 + lane, a.Sq - 1);
@@ -850,13 +852,14 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
         typename E::V4 ov = {t0[0], t0[1], t1[0], t1[1]};
         *reinterpret_cast<ACCT_LDS typename E::V4*>(obuf + l32 * OPITCH + (32 * db + 8 * r4 + 4 * g) * 2) = ov;
       }
-    constexpr int NCH = C::CPR;
+    const int nch = a.hd >> 3;                       // valid 16-byte chunks per row
+    const uint32_t nch_inv = recip16(nch);
 #pragma unroll
-    for (int i = 0; i < (32 * NCH + 63) / 64; i++) {
+    for (int i = 0; i < (32 * C::CPR + 63) / 64; i++) {
       const int idx = lane + 64 * i;
-      const int r = idx / NCH, ch = idx % NCH;
+      const int r = div_small(idx, nch_inv), ch = idx - r * nch;
       const int grow = wk0 + 32 * gk + r;
-      if (idx < 32 * NCH && grow < a.Sk) {
+      if (idx < 32 * nch && grow < a.Sk) {
         const u32x4 v = *reinterpret_cast<const ACCT_LDS u32x4*>(obuf + r * OPITCH + ch * 16);
         *reinterpret_cast<u32x4*>(outp + (int64_t)grow * oss + ch * 8) = v;
       }
@@ -926,7 +929,8 @@ bool launch_variants_complete() { return false; }
 bool launch_variants_complete() { return fwd_variants_complete(); }
 #endif
 
-hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t st) {
+hipError_t launch_bwd(const FaArgs& a, int dtype, int Dr, int stages, hipStream_t st) {
+  const int D = head_dim_class(Dr);
 #ifdef ACCT_DEV_BUILD
   if (dtype != 0 || D != 128) return hipErrorNotSupported;
   return launch_bwd_d<f16, 128>(a, stages, st);

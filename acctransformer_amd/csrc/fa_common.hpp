@@ -112,6 +112,7 @@ struct FaArgs {
   const uint32_t* colbits;             // [MB, Tr, Sk, 4] dense mask of the 'apply' blocks packed by key column: bit r of the
                                        // 128-bit entry = mask[128*qb + r][key] (dK/dV kernel); may be null
   int B, N, Sq, Sk;
+  int hd;                              // head dim (<= the kernel's template head dim, a multiple of 8): columns past it do not exist
   int Tr, Tc;                          // number of 128-row / 128-column blocks
   int64_t q_sb, q_sh, q_ss;
   int64_t k_sb, k_sh, k_ss;
@@ -282,11 +283,11 @@ template <int D> struct SwzCfg {
 
 // Stage rows [row0, row0 + ROWS) of a row-major global matrix into a swizzled LDS
 // tile with NW waves.  Rows past nrows repeat the last valid row (finite data whose
-// contribution is zeroed by the caller's masking), slots past the valid chunks
-// repeat the last valid chunk.
+// contribution is zeroed by the caller's masking), slots past the `cpr` valid 16-byte
+// chunks of a row (head dim / 8) repeat the last valid chunk.
 // `wv` < 0: the NW waves are the workgroup's first NW; else the calling wave's index among the NW.
 template <typename T, int D, int ROWS, int NW>
-ACCT_DEV void tile_dma(const T* base, int64_t row_stride, int row0, int nrows, ACCT_LDS char* buf, int wv = -1) {
+ACCT_DEV void tile_dma(const T* base, int64_t row_stride, int row0, int nrows, ACCT_LDS char* buf, int cpr, int wv = -1) {
   using C = SwzCfg<D>;
   constexpr int NI = ROWS / C::RPI;
   static_assert(NI % NW == 0, "tile rows must split evenly over the waves");
@@ -297,7 +298,7 @@ ACCT_DEV void tile_dma(const T* base, int64_t row_stride, int row0, int nrows, A
   for (int i = 0; i < NI / NW; i++) {
     const int inst = wave * (NI / NW) + i;
     const int r = inst * C::RPI + lane / C::CH;
-    const int lc = min((lane % C::CH) ^ C::swz(r), C::CPR - 1);
+    const int lc = min((lane % C::CH) ^ C::swz(r), cpr - 1);
     const int grow = min(row0 + r, nrows - 1);
     const T* src = base + (int64_t)grow * row_stride + lc * 8;
     // Issued as inline assembly on purpose: the compiler then does not order every later LDS read
@@ -326,21 +327,21 @@ struct TileDma {
   uint32_t voff[NV];
   uint32_t lds0;                                   // LDS byte offset of this wave's first 1 KB slab within a tile
   // `wv` < 0: the NW waves are the workgroup's first NW; else the calling wave's index among the NW
-  ACCT_DEV void plan(int64_t row_stride, int wv = -1) {
+  ACCT_DEV void plan(int64_t row_stride, int cpr, int wv = -1) {
     static_assert(NI % NW == 0, "tile rows must split evenly over the waves");
     const int lane = threadIdx.x & 63, wave = wv < 0 ? (int)(threadIdx.x >> 6) : wv;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       const int inst = wave * NIW + i;
       const int r = inst * C::RPI + lane / C::CH;
-      const int lc = min((lane % C::CH) ^ C::swz(r), C::CPR - 1);
+      const int lc = min((lane % C::CH) ^ C::swz(r), cpr - 1);
       voff[i] = (uint32_t)((r * row_stride + lc * 8) * (int64_t)sizeof(T));
     }
     lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(wave * NIW * 1024));
   }
   // plan-free variant for kernels without registers to spare: the 32-bit offsets are re-derived
   // (a few 32-bit vector ops per instruction); rows [row0, row0 + ROWS) must exist
-  static ACCT_DEV void issue_direct(const T* base, int64_t row_stride, int row0, ACCT_LDS char* buf) {
+  static ACCT_DEV void issue_direct(const T* base, int64_t row_stride, int row0, ACCT_LDS char* buf, int cpr) {
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));
     const int lane = tid & 63, wave = tid >> 6;
@@ -356,7 +357,7 @@ struct TileDma {
 #pragma unroll
     for (int i = 0; i < NIW; i++) {
       const int r = (wave * NIW + i) * C::RPI + lane / C::CH;
-      const int lc = min((lane % C::CH) ^ C::swz(r), C::CPR - 1);
+      const int lc = min((lane % C::CH) ^ C::swz(r), cpr - 1);
       const uint32_t voff = (uint32_t)r * rs + (uint32_t)lc * 16u;
       asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(tile), "s"(dst0 + i * 1024)
                    : "memory");
@@ -440,6 +441,10 @@ struct DropRowStage {
   }
 };
 
+
+// idx / n for idx < 1024 and n <= 32 (the epilogues' chunk index -> row): exact with a 16-bit reciprocal
+ACCT_DEV int div_small(int idx, uint32_t inv16) { return (int)(((uint32_t)idx * inv16) >> 16); }
+ACCT_DEV uint32_t recip16(int n) { return (65536u + (uint32_t)n - 1u) / (uint32_t)n; }
 
 // byte offset of logical chunk `lc` in a row whose swz3(row) is `swz`
 ACCT_DEV int swz_off(int lc, int swz) { return (lc ^ swz) << 4; }

@@ -76,9 +76,9 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
     const int row = min(wq0 + 32 * gq + l32, a.Sq - 1);     // rows past Sq repeat the last row; never stored
 #pragma unroll
     for (int t = 0; t < C::KS; t++) {
-      // D % 16 == 8: the upper half of the last k-step lies past the row; zeros there make the products
-      // ignore whatever the K tile holds in that slot
-      const bool inside = (D % 16 == 0) || 16 * t + 8 * g < D;
+      // k-steps (or the upper half of one) past the head dim: zeros there make the products ignore whatever
+      // the K tile holds in those slots
+      const bool inside = 16 * t + 8 * g < a.hd;
       V8 z;
 #pragma unroll
       for (int e = 0; e < 8; e++) z[e] = 0;
@@ -126,8 +126,9 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   const bool alibi_vec = BIAS && (((uintptr_t)a.alibi & 7) | ((a.al_sb | a.al_sh | a.al_sq) & 3)) == 0;
 
   TileDma<T, D, BN, NW> kdma, vdma;
-  kdma.plan(a.k_ss);
-  vdma.plan(a.v_ss);
+  const int cpr = a.hd >> 3;                                // valid 16-byte chunks per row
+  kdma.plan(a.k_ss, cpr);
+  vdma.plan(a.v_ss, cpr);
   // bias tiles of this wave's rows are staged through a wave-private LDS region one tile ahead
   ACCT_LDS char* bias_lds = smem + 4 * TILEB + wave * (QG * 4096);
   const bool bias_staged = BIAS && (a.Sk & 7) == 0 && (((uintptr_t)a.alibi & 15) | ((a.al_sb | a.al_sh | a.al_sq) & 7)) == 0;
@@ -165,7 +166,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   // stage key rows [j BN, (j+1) BN) of K or V into an LDS tile
   auto stage_tile = [&](const TileDma<T, D, BN, NW>& dma, const T* base, int64_t ss, int j, ACCT_LDS char* dst) {
     if ((j + 1) * BN <= a.Sk) dma.issue(base, ss, j * BN, dst);
-    else tile_dma<T, D, BN, NW>(base, ss, j * BN, a.Sk, dst);   // ragged last tile: clamped rows
+    else tile_dma<T, D, BN, NW>(base, ss, j * BN, a.Sk, dst, cpr);   // ragged last tile: clamped rows
   };
   // S^T = K Q^T : s[gq][c] is the 32(kv) x 32(q) tile of kv chunk c
   auto gemm_s = [&](const ACCT_LDS char* kbuf, f32x16 (&s)[QG][KT]) {
@@ -348,8 +349,8 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   };
 
   if (j_lo <= j_hi) {
-    tile_dma<T, D, BN, NW>(kp, a.k_ss, j_lo * BN, a.Sk, smem);
-    tile_dma<T, D, BN, NW>(vp, a.v_ss, j_lo * BN, a.Sk, smem + TILEB);
+    tile_dma<T, D, BN, NW>(kp, a.k_ss, j_lo * BN, a.Sk, smem, cpr);
+    tile_dma<T, D, BN, NW>(vp, a.v_ss, j_lo * BN, a.Sk, smem + TILEB, cpr);
     if (BIAS && bias_staged && wq0 < a.Sq) stage_bias(j_lo);
     DropStage::issue(a, bh, wq0, j_lo, lane, drop_lds);
     // A full wait the compiler can see: every load issued so far (Q fragments included) is complete, so
@@ -404,13 +405,14 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
         *reinterpret_cast<ACCT_LDS typename E::V4*>(obuf + l32 * OPITCH + (32 * db + 8 * r4 + 4 * g) * 2) = ov;
       }
     // read back row-contiguous: 16-byte chunk ch of row r
-    constexpr int NCH = C::CPR;                      // valid chunks per row
+    const int nch = a.hd >> 3;                       // valid 16-byte chunks per row
+    const uint32_t nch_inv = recip16(nch);
 #pragma unroll
-    for (int i = 0; i < (32 * NCH + 63) / 64; i++) {
+    for (int i = 0; i < (32 * C::CPR + 63) / 64; i++) {
       const int idx = lane + 64 * i;
-      const int r = idx / NCH, ch = idx % NCH;
+      const int r = div_small(idx, nch_inv), ch = idx - r * nch;
       const int grow = wq0 + 32 * gq + r;
-      if (idx < 32 * NCH && grow < a.Sq) {
+      if (idx < 32 * nch && grow < a.Sq) {
         const u32x4 v = *reinterpret_cast<const ACCT_LDS u32x4*>(obuf + r * OPITCH + ch * 16);
         *reinterpret_cast<u32x4*>(op + (int64_t)grow * a.o_ss + ch * 8) = v;
       }
@@ -470,7 +472,8 @@ bool fwd_variants_complete() { return false; }
 bool fwd_variants_complete() { return true; }
 #endif
 
-hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st) {
+hipError_t launch_fwd(const FaArgs& a, int dtype, int Dr, int qg, hipStream_t st) {
+  const int D = head_dim_class(Dr);
 #ifdef ACCT_DEV_BUILD
   if (dtype != 0 || D != 128) return hipErrorNotSupported;
   return launch_fwd_d<f16, 128>(a, qg, st);

@@ -22,6 +22,14 @@ inline hipError_t allow_dynamic_lds(const void* kern, size_t bytes) {
   return e;
 }
 
+// The kernels are built for the head dims 40, 64, 80, 128, 160 and 256.  Any other multiple of 8 runs on the next
+// built size of its row layout (128-, 256- or 512-byte LDS rows): the columns past the head dim are never loaded
+// as operands (zero fragments) and never stored.
+inline int head_dim_class(int D) {
+  if (D == 40 || D == 80 || D == 160) return D;
+  return D <= 64 ? 64 : (D <= 128 ? 128 : 256);
+}
+
 // forward: variant 3 = 8 waves x 32 query rows, 1 = 4 waves x 32 rows; the bias / dropout
 // variants are picked from a.alibi / a.droprow
 hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st);

@@ -37,7 +37,9 @@ extern "C" {
 #define ACCT_E_NULLPTR  (-1)   /* a required pointer is NULL */
 #define ACCT_E_SHAPE    (-2)   /* non-positive or inconsistent extent / stride */
 #define ACCT_E_DTYPE    (-3)   /* dtype is neither ACCT_F16 nor ACCT_BF16 */
-#define ACCT_E_HEADDIM  (-4)   /* D unsupported (built: 40, 64, 80, 128, 160, 256; 40, 160 and 256 without bias and dropout) */
+#define ACCT_E_HEADDIM  (-4)   /* D unsupported: not a multiple of 8, above 256 (L/flash_attention.py:26,105-106), or 40 / above 128 together
+                                  with a bias or dropout (kernels are built for 40, 64, 80, 128, 160, 256; other
+                                  multiples of 8 run on the next built size) */
 #define ACCT_E_ARCH     (-5)   /* current device is not gfx950 */
 #define ACCT_E_LAUNCH   (-6)   /* HIP reported a launch error */
 #define ACCT_E_WORKSPACE (-7)  /* workspace missing or too small */

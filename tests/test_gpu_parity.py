@@ -616,6 +616,31 @@ def test_extra_head_dims_with_masks(D, dtype):
     assert e.value.code == -4
 
 
+def test_head_dims_between_the_built_sizes():
+    # any multiple of 8 up to 256 (the reference's layer takes head dims up to 256,
+    # nn/layer/flash_attention.py:26,105-106): sizes that are not built run on the next built size of their row
+    # layout, the columns past the head dim never loaded as operands and never stored
+    for D, dtype, extra in ((96, torch.float16, "drop"), (32, torch.float16, "bias"), (112, torch.bfloat16, None),
+                            (192, torch.float16, None), (144, torch.float16, None), (8, torch.float16, None)):
+        B, N, Sq, Sk = 1, 2, 200, 333
+        tol = dict(atol=ATOL_BF16, rtol=RTOL_BF16) if dtype == torch.bfloat16 else {}
+        q, k, v, dO = (_gen(s, 870 + i + D, dtype) for i, s in enumerate([(B, N, Sq, D), (B, N, Sk, D), (B, N, Sk, D), (B, N, Sq, D)]))
+        rng = np.random.default_rng(D)
+        mask = (rng.random((B, Sq, Sk)) < 0.3).astype(np.uint8)
+        mask[:, :, 0] = 0
+        okw, kw = dict(scale=D ** -0.5, attn_mask=mask), dict(scale=D ** -0.5, mask_kind=_capi.MASK_DENSE_U8, attn_mask=mask)
+        if extra == "drop":
+            d8 = (rng.random((B, N, Sq, Sk)) < 0.8).astype(np.uint8)
+            okw.update(drop_mask=d8, keep_prob=0.8); kw.update(drop_mask=d8, keep_prob=0.8)
+        if extra == "bias":
+            al = (0.05 * torch.randn(1, N, 1, Sk, generator=torch.Generator().manual_seed(D))).to(dtype)
+            okw.update(alibi=al.float().numpy()); kw.update(alibi=al)
+        res = _run(q, k, v, dO, **kw)
+        _check_all(q, k, v, dO, okw, res, **tol)
+        # the output rows are exactly D wide: nothing was written past them (the next row would be damaged)
+        assert res[0].shape[-1] == D and torch.isfinite(res[0].float()).all()
+
+
 @pytest.mark.parametrize("D, Sq, Sk", [(40, 4096, 4096), (40, 4096, 77), (80, 1024, 77), (160, 256, 256), (160, 64, 77), (160, 1024, 1024)])
 def test_wukong_training_shapes(D, Sq, Sk):
     # the sequence lengths and head dims the reference's wukong tiling strategy is written for (self attention at
