@@ -222,11 +222,16 @@ def main():
             oo, ll = torch.empty_like(qq), torch.empty(qq.shape[:3], dtype=torch.float32, device=dev)
             g3 = [torch.empty_like(t) for t in (qq, kk, vv)]
             pp.o_stride = _capi._bhs_strides(oo)
+            # with dropout, the forward call packs (or draws) the keep bits into a buffer that the backward call of
+            # the same step reads (drop_bits / drop_bits_filled of the C ABI), as the Python operator does
+            bits = _capi.attach_drop_bits(pp, dev)
             nw = max(lib.acct_fa_bwd_workspace_bytes(P(pp)), lib.acct_fa_fwd_workspace_bytes(P(pp)), 256)
             w = torch.empty(nw, dtype=torch.uint8, device=dev)
 
             def one():
+                pp.drop_bits_filled = 0
                 check(lib.acct_fa_fwd(P(pp), oo.data_ptr(), ll.data_ptr(), w.data_ptr(), nw, st))
+                pp.drop_bits_filled = 1 if bits is not None else 0
                 check(lib.acct_fa_bwd(P(pp), oo.data_ptr(), dd.data_ptr(), ll.data_ptr(), g3[0].data_ptr(), g3[1].data_ptr(),
                                       g3[2].data_ptr(), w.data_ptr(), nw, st))
             for _ in range(3):
