@@ -27,8 +27,9 @@ Differences from the reference Cell that a caller can see:
     state: a forward that is re-run (activation checkpointing) would draw a
     new mask.  Pass `dropout_state=(seed, offset)` to `forward` to fix the
     stream of a call explicitly; the same pair reproduces the same mask.
-  * Head dims built: 40, 64, 80, 128, 160, 256 (the reference admits any
-    multiple of 16 up to 256); others raise when the op is called.
+  * Head dims: any multiple of 8 up to 256 (the reference admits multiples
+    of 16 up to 256); others raise when the op is called.  alibi_mask and
+    dropout need a head_dim of at most 128 other than 40.
 """
 from __future__ import annotations
 
