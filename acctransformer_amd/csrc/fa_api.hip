@@ -89,6 +89,12 @@ int validate(const acct_fa_params* p, bool backward) {
   if (p->dtype != ACCT_F16 && p->dtype != ACCT_BF16) return fail(ACCT_E_DTYPE, "dtype %d is neither ACCT_F16 nor ACCT_BF16", p->dtype);
   if (p->B <= 0 || p->N <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->D <= 0)
     return fail(ACCT_E_SHAPE, "extents must be positive: B=%d N=%d Sq=%d Sk=%d D=%d", p->B, p->N, p->Sq, p->Sk, p->D);
+  {
+    // grid sizes and (batch*head, tile) indices are 32-bit in the kernels
+    const int64_t smax = p->Sq > p->Sk ? p->Sq : p->Sk;
+    if ((int64_t)p->B * p->N > 0x7fffffff || (int64_t)p->B * p->N * ((smax + 31) / 32) > 0x7fffffff)
+      return fail(ACCT_E_SHAPE, "B*N*ceil(S/32) must stay below 2^31: B=%d N=%d Sq=%d Sk=%d", p->B, p->N, p->Sq, p->Sk);
+  }
   if (p->D > 256) return fail(ACCT_E_HEADDIM, "head_dim too large, reduce head_dim and try again. (D=%d > 256)", p->D);
   if (p->D % 8 != 0) return fail(ACCT_E_HEADDIM, "head_dim %d is not a multiple of 8", p->D);
   (void)backward;

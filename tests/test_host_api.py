@@ -63,7 +63,7 @@ def _params(**over):
 @pytest.mark.parametrize("over, code", [
     (dict(dtype=7), -3), (dict(B=0), -2), (dict(D=512), -4), (dict(D=100), -4), (dict(scale=0.0), -8),
     (dict(keep_prob=1.5), -8), (dict(prev_block_num=-1), -8), (dict(mask_kind=6), -8), (dict(mask_kind=_capi.MASK_DENSE_F16), -1),
-    (dict(drop_mask_kind=2), -8),
+    (dict(drop_mask_kind=2), -8), (dict(B=1 << 20, N=1 << 12), -2), (dict(B=1 << 15, N=1 << 10, Sq=1 << 16), -2),
     (dict(mask_kind=_capi.MASK_DENSE_U8), -1), (dict(row_block_prefix=100), -8), (dict(q=None), -1),
 ])
 def test_validation_error_codes(over, code):
