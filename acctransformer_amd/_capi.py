@@ -92,6 +92,8 @@ def load():
     I64P = ctypes.POINTER(ctypes.c_int64)
     lib.acct_fa_infer_shape.argtypes = [I64P, ctypes.c_int, I64P, ctypes.c_int, I64P, ctypes.c_int, I64P]
     lib.acct_fa_infer_shape.restype = ctypes.c_int
+    lib.acct_probe_mfma_rate.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
+    lib.acct_probe_mfma_rate.restype = ctypes.c_int
     lib.acct_version.argtypes = []
     lib.acct_version.restype = ctypes.c_int
     _lib = lib

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define ACCT_FA_VERSION 104
+#define ACCT_FA_VERSION 105
 
 /* error codes (0 = success) */
 #define ACCT_OK          0
@@ -198,6 +198,14 @@ int acct_version(void);
  * that was compiled with a reduced variant set (such a build refuses the calls it cannot serve with
  * ACCT_E_LAUNCH).  No counterpart in the reference: a guard for packaging and tests. */
 int acct_build_is_complete(void);
+
+/* Measurement aid, no counterpart in the reference: the rate (TFLOP/s, whole GPU) at which the current device
+ * retires back-to-back independent v_mfma_f32_32x32x16_f16 from registers, two waves per SIMD on every CU and
+ * nothing else running -- the ceiling of any fp16 kernel built on that instruction.  varying_operands != 0:
+ * operands differ from lane to lane as real data does; 0: one value in every lane (the clock, and with it the
+ * rate, depends on how much the operands toggle).  Runs about 0.1 s of kernels on `stream` and waits for them.
+ * bench.py reports both figures beside the attention kernels' roofline fraction. */
+int acct_probe_mfma_rate(int varying_operands, double* tflops, void* stream);
 
 #ifdef __cplusplus
 }

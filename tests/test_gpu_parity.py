@@ -892,6 +892,22 @@ def test_cpu_sized_configuration_b1_n4_s512_d64():
     assert verdict == "Pass", (over, over_max)
 
 
+def test_mfma_rate_probe_reports_a_plausible_ceiling():
+    # the register-only MFMA loop that bench.py reports beside the roofline fraction: a rate between a fifth
+    # of the nominal dense fp16 peak and the peak itself, and not lower with identical operands in every lane
+    # than with operands that toggle (a generous band: the clock differs from box to box)
+    lib = _capi.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rates = []
+    for varying in (1, 0):
+        r = ctypes.c_double(0.0)
+        assert lib.acct_probe_mfma_rate(varying, ctypes.byref(r), st) == 0, lib.acct_last_error().decode()
+        rates.append(r.value)
+    assert 500.0 < rates[0] <= 2516.6 * 1.02, rates
+    assert rates[1] >= 0.95 * rates[0], rates
+    assert lib.acct_probe_mfma_rate(1, None, st) == -1
+
+
 # ---- both branches of the workgroup map (more / not more than 64 batch*head pairs) -------------------
 def test_slice_equivalence_across_the_workgroup_map_branches():
     # B*N = 256 takes the XCD-grouped launch order, each slice of 64 the plain one: every (batch, head) pair must
