@@ -150,10 +150,13 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   // bias tiles of this wave's rows are staged through a wave-private LDS region one tile ahead
   ACCT_LDS char* bias_lds = smem + 4 * TILEB + wave * (QG * 4096);
   const bool bias_staged = BIAS && (a.Sk & 7) == 0 && (((uintptr_t)a.alibi & 15) | ((a.al_sb | a.al_sh | a.al_sq) & 7)) == 0;
+  const bool row_bias = BIAS && a.al_sq == 0;            // the bias depends on the key only: one 128-byte row per tile
   auto stage_bias = [&](int jn) {
 #pragma unroll
-    for (int gq = 0; gq < QG; gq++)
-      bias_tile_dma<T>(alibip, a.al_sq, wq0 + 32 * gq, a.Sq, jn * 64, a.Sk, bias_lds + gq * 4096);
+    for (int gq = 0; gq < QG; gq++) {
+      if (row_bias) bias_row_dma<T>(alibip, jn * 64, a.Sk, bias_lds + gq * 4096);
+      else bias_tile_dma<T>(alibip, a.al_sq, wq0 + 32 * gq, a.Sq, jn * 64, a.Sk, bias_lds + gq * 4096);
+    }
   };
   // keep bits of this wave's rows and one tile, staged with the tile's DMA (double buffered)
   using DropStage = DropRowStage<DROP, QG, 2>;
@@ -215,7 +218,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
               // q.k): nothing per score afterwards, no bias registers alive next to the scores
               typename E::V4 bv[4];
 #pragma unroll
-              for (int r4 = 0; r4 < 4; r4++) bv[r4] = bias_tile_read<T>(bias_lds + gq * 4096, l32, 4 * c + r4, g);
+              for (int r4 = 0; r4 < 4; r4++) bv[r4] = bias_tile_read<T>(bias_lds + gq * 4096, row_bias ? 0 : l32, 4 * c + r4, g);
 #pragma unroll
               for (int r = 0; r < 16; r++) s[gq][r] = (float)bv[r >> 2][r & 3] * a.inv_scale;
             } else {
@@ -558,7 +561,15 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     }
   };
 
-  const bool bias_staged = BIAS && !krole && wk0 < a.Sk && (a.Sk & 7) == 0 &&
+  // A bias with row stride 0 (the reference's ALiBi form [B, N, 1, Sk]) depends on the key only: a lane of this
+  // kernel owns a key column, so the bias is one value per lane and key group for the whole query loop
+  // (in units of the raw scores; 0 for the K role, whose accumulators hold dP)
+  const bool row_bias = BIAS && a.al_sq == 0;
+  float brow[NGK];
+#pragma unroll
+  for (int gk = 0; gk < NGK; gk++)
+    brow[gk] = (row_bias && !krole) ? (float)alibip[min(wk0 + 32 * gk + l32, a.Sk - 1)] * a.inv_scale : 0.f;
+  const bool bias_staged = BIAS && !row_bias && !krole && wk0 < a.Sk && (a.Sk & 7) == 0 &&
                            (((uintptr_t)a.alibi & 15) | ((a.al_sb | a.al_sh | a.al_sq) & 7)) == 0;
   auto stage_bias = [&](int cn) { bias_tile_dma<T, false>(alibip, a.al_sq, cn * 32, a.Sq, wk0, a.Sk, bias_lds); };
 
@@ -621,7 +632,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
       if (cidx >= c_lo && cidx <= c_hi) {
         const uint32_t cls = classify(cidx, flwin.get(cidx >> 2, lane));
         const bool act = cls & 1u, apply_mask = cls & 2u, limits = cls & 4u, diag = cls & 8u;
-        const bool edge = (BIAS && !bias_staged) || apply_mask || limits;   // (a staged bias is already inside the scores)
+        const bool edge = (BIAS && !bias_staged && !row_bias) || apply_mask || limits;   // (a staged or per-key bias is already inside the scores)
         if (act) {
           const int c = cidx & 1, qc0 = cidx * 32;
           // Where the registers do not allow keeping them (see above), the per-lane LDS offsets are
@@ -668,7 +679,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 #pragma unroll
             for (int gk = 0; gk < NGK; gk++)
 #pragma unroll
-              for (int r = 0; r < 16; r++) t0[gk][r] = 0.f;
+              for (int r = 0; r < 16; r++) t0[gk][r] = BIAS ? brow[gk] : 0.f;
           }
           {
             // software pipeline: the A fragments travel through a ring of ARING register sets (ARING reads in
@@ -710,7 +721,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
               // passes that each keep few values live: + bias/scale (unstaged bias only); - 10000/scale where the mask bit of
               // (row, key) is set; -inf where the key comes after the query (causal) or where the key
               // or the query row does not exist (the probability is exactly 0 either way).
-              if (BIAS && !bias_staged) {                   // a bias the DMA cannot stage (alignment): direct loads
+              if (BIAS && !bias_staged && !row_bias) {      // a bias the DMA cannot stage (alignment): direct loads
                 const int qlast = a.Sq - 1 - qc0;               // last valid row, relative to the chunk
                 const T* brow0 = alibip + (int64_t)qc0 * a.al_sq;
 #pragma unroll

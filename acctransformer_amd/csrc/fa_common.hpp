@@ -419,6 +419,17 @@ ACCT_DEV void dma4(const void* src, ACCT_LDS char* dst) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(d) : "memory");
 }
 
+// A bias that depends on the key only (row stride 0, the reference's ALiBi form): the values of the keys
+// kv0 .. kv0 + 127, one dword (two keys) per lane, land as row 0 of the region bias_tile_read reads (the
+// chunks of row 0 are not swizzled), so a reader passes row 0 instead of its own.  Same requirements as
+// bias_tile_dma; keys past Sk repeat the last pair.
+template <typename T>
+ACCT_DEV void bias_row_dma(const T* base, int kv0, int Sk, ACCT_LDS char* dst) {
+  int ln = threadIdx.x & 63;
+  asm volatile("" : "+v"(ln));
+  dma4(base + min(kv0 + 2 * ln, Sk - 2), dst);
+}
+
 // Keep-bit words (dropout, packed by query row) of the 32*QG rows of a wave and the KT 32-key chunks of one
 // K/V tile, brought into a wave-private LDS buffer [row][KT] by DMA together with the tile.  Read from LDS
 // in the tile loop, they need no wait on the vector-memory counter, which would also wait for the K/V

@@ -132,10 +132,13 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   // bias tiles of this wave's rows are staged through a wave-private LDS region one tile ahead
   ACCT_LDS char* bias_lds = smem + 4 * TILEB + wave * (QG * 4096);
   const bool bias_staged = BIAS && (a.Sk & 7) == 0 && (((uintptr_t)a.alibi & 15) | ((a.al_sb | a.al_sh | a.al_sq) & 7)) == 0;
+  const bool row_bias = BIAS && a.al_sq == 0;              // the bias depends on the key only: one 128-byte row per tile
   auto stage_bias = [&](int jn) {
 #pragma unroll
-    for (int gq = 0; gq < QG; gq++)
-      bias_tile_dma<T>(alibip, a.al_sq, wq0 + 32 * gq, a.Sq, jn * 64, a.Sk, bias_lds + gq * 4096);
+    for (int gq = 0; gq < QG; gq++) {
+      if (row_bias) bias_row_dma<T>(alibip, jn * 64, a.Sk, bias_lds + gq * 4096);
+      else bias_tile_dma<T>(alibip, a.al_sq, wq0 + 32 * gq, a.Sq, jn * 64, a.Sk, bias_lds + gq * 4096);
+    }
   };
   // keep bits of this wave's rows and one tile, staged with the tile's DMA (double buffered)
   using DropStage = DropRowStage<DROP, QG, KT>;
@@ -234,7 +237,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
 #pragma unroll
           for (int c = 0; c < 2; c++)
 #pragma unroll
-            for (int r4 = 0; r4 < 4; r4++) bv[c][r4] = bias_tile_read<T>(bias_lds + gq * 4096, l32, 4 * c + r4, g);
+            for (int r4 = 0; r4 < 4; r4++) bv[c][r4] = bias_tile_read<T>(bias_lds + gq * 4096, row_bias ? 0 : l32, 4 * c + r4, g);
           if (gq == QG - 1) {
             // the tile is in registers: its LDS region can take the next tile, which has the rest of
             // this step to land (the end-of-step wait covers it)

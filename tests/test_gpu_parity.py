@@ -307,6 +307,30 @@ def test_all_side_inputs_ragged(dtype, Sq, Sk, D):
                                       drop_mask=drop, keep_prob=0.85, alibi=al), **tol)
 
 
+@pytest.mark.parametrize("dtype, Sq, Sk, D", [(torch.float16, 333, 328, 128), (torch.float16, 200, 333, 128),
+                                              (torch.bfloat16, 300, 456, 64), (torch.float16, 520, 392, 80)])
+def test_key_only_bias_with_all_side_inputs(dtype, Sq, Sk, D):
+    # the reference's ALiBi form [B, N, 1, Sk] (row stride 0, here different per batch and head) together with a
+    # dense mask and dropout: the kernels stage one bias row per tile (forward, dQ) or keep one value per lane
+    # (dK/dV) instead of a tile; lengths with and without the Sk % 8 == 0 that the staging needs
+    B, N = 2, 3
+    q, dO = (_gen((B, N, Sq, D), s, dtype) for s in (171, 174))
+    k, v = (_gen((B, N, Sk, D), s, dtype) for s in (172, 173))
+    rng = np.random.default_rng(175)
+    mask = (rng.random((B, Sq, Sk)) < 0.25).astype(np.uint8)
+    mask[:, :, 0] = 0
+    drop = (rng.random((B, N, Sq, Sk)) < 0.85).astype(np.uint8)
+    al = (0.5 * torch.randn((B, N, 1, Sk), generator=torch.Generator().manual_seed(176))).to(dtype)
+    tol = dict(atol=2e-2, rtol=1e-2) if dtype == torch.bfloat16 else {}
+    okw = dict(scale=D ** -0.5, attn_mask=mask, drop_mask=drop, keep_prob=0.85, alibi=al.float().numpy())
+    _check_all(q, k, v, dO, okw, _run(q, k, v, dO, scale=D ** -0.5, mask_kind=_capi.MASK_DENSE_U8, attn_mask=mask,
+                                      drop_mask=drop, keep_prob=0.85, alibi=al), **tol)
+    # without the other side inputs, causal by index compare
+    tri = np.triu(np.ones((1, Sq, Sk), np.uint8), 1)
+    okw = dict(scale=D ** -0.5, attn_mask=tri, alibi=al.float().numpy())
+    _check_all(q, k, v, dO, okw, _run(q, k, v, dO, scale=D ** -0.5, mask_kind=_capi.MASK_CAUSAL, alibi=al), **tol)
+
+
 @pytest.mark.parametrize("form", ["row_bias", "full_bias"])
 def test_alibi_forms(form):
     B, N, S, D = 1, 8, 1024, 128
