@@ -20,7 +20,7 @@ namespace acct {
 
 template <typename T, int D, int QG, int NW, bool BIAS, bool DROP, bool MASKT, int KT = 2>
 __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
-  static_assert(KT == 2 || (KT == 4 && !BIAS), "key tiles are 64 rows, or 128 rows in the variants without bias");
+  static_assert(KT == 2 || KT == 4, "key tiles are 64 or 128 rows (with a bias, 128 rows take the key-only form of it only)");
   constexpr int BN = 32 * KT;                       // key rows per tile
   constexpr int FRING = 4, VRING = 3;   // fragment reads in flight ahead of their MFMA (K row-major / V transposed)
   constexpr int TPB = 128 / BN;                     // tiles per 128-column block
@@ -115,8 +115,15 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   // Scores stay in raw q.k units (exp2 argument = s * scale*log2e - m * scale*log2e, one FMA) unless a
   // bias is added, in which case they become scale*s + bias first (one mixed-precision FMA per score:
   // the fp16 / bf16 bias is an operand as it is).
-  const float cmul = BIAS ? kLog2e : a.scale_log2e;
-  const float madd = BIAS ? kMaskFill : a.mask_add_raw;            // the additive -10000 in the units of s
+  // A key-only bias (row stride 0) that the DMA can stage goes in as the INITIAL value of the score accumulators
+  // instead (bias / scale, the MFMAs add q.k): the scores stay in raw units and nothing is spent per score.
+  const bool bias_staged = BIAS && (a.Sk & 7) == 0 && (((uintptr_t)a.alibi & 15) | ((a.al_sb | a.al_sh | a.al_sq) & 7)) == 0;
+  // (the launcher picks 128-key tiles for a bias only when both hold: known at compile time there)
+  const bool row_bias = BIAS && (KT == 4 || a.al_sq == 0);   // the bias depends on the key only: one row per tile
+  const bool acc_bias = BIAS && (KT == 4 || (row_bias && bias_staged));
+  const bool scaled = BIAS && !acc_bias;                   // scores are turned into scale*s + bias before the softmax
+  const float cmul = scaled ? kLog2e : a.scale_log2e;
+  const float madd = scaled ? kMaskFill : a.mask_add_raw;          // the additive -10000 in the units of s
   const float lazy_thr = 8.0f / cmul;                              // 8 octaves, in the units of s
   const int mb = a.mask_sb ? b : 0;
   const uint8_t* maskp = a.mask ? a.mask + (a.mask_kind == kMaskDense ? (int64_t)mb * a.mask_sb * a.mask_es : 0) : nullptr;
@@ -130,19 +137,22 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   kdma.plan(a.k_ss, cpr);
   vdma.plan(a.v_ss, cpr);
   // bias tiles of this wave's rows are staged through a wave-private LDS region one tile ahead
-  ACCT_LDS char* bias_lds = smem + 4 * TILEB + wave * (QG * 4096);
-  const bool bias_staged = BIAS && (a.Sk & 7) == 0 && (((uintptr_t)a.alibi & 15) | ((a.al_sb | a.al_sh | a.al_sq) & 7)) == 0;
-  const bool row_bias = BIAS && a.al_sq == 0;              // the bias depends on the key only: one 128-byte row per tile
+  // (with 128-key tiles only the key-only form is served: two 256-byte rows per wave)
+  constexpr int BIASB = BIAS ? (KT == 4 ? 512 : QG * 4096) : 0;
+  static_assert(KT == 2 || !BIAS || QG == 1, "128-key tiles with a bias: 32 rows per wave");
+  ACCT_LDS char* bias_lds = smem + 4 * TILEB + wave * BIASB;
+  // (a key-only bias: rows of consecutive tiles alternate between two 256-byte slots of the region, so the next
+  // one is requested together with the next K/V tile; a tile bias has one slot and is requested once read)
   auto stage_bias = [&](int jn) {
 #pragma unroll
     for (int gq = 0; gq < QG; gq++) {
-      if (row_bias) bias_row_dma<T>(alibip, jn * 64, a.Sk, bias_lds + gq * 4096);
+      if (row_bias) bias_row_dma<T>(alibip, jn * BN, a.Sk, bias_lds + gq * 4096 + (acc_bias ? (jn & 1) * 256 : 0));
       else bias_tile_dma<T>(alibip, a.al_sq, wq0 + 32 * gq, a.Sq, jn * 64, a.Sk, bias_lds + gq * 4096);
     }
   };
   // keep bits of this wave's rows and one tile, staged with the tile's DMA (double buffered)
   using DropStage = DropRowStage<DROP, QG, KT>;
-  ACCT_LDS char* drop_lds = smem + 4 * TILEB + (BIAS ? NW * QG * 4096 : 0) + wave * (2 * DropStage::BYTES);
+  ACCT_LDS char* drop_lds = smem + 4 * TILEB + NW * BIASB + wave * (2 * DropStage::BYTES);
   // ---- the phases of a tile step: classification, S^T = K Q^T, online softmax, O^T += V^T P^T ----
   const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
   BlkClassWindow flwin;                                      // block classes of a dense mask: 64 blocks at a time in scalar registers
@@ -172,13 +182,27 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
     else tile_dma<T, D, BN, NW>(base, ss, j * BN, a.Sk, dst, cpr);   // ragged last tile: clamped rows
   };
   // S^T = K Q^T : s[gq][c] is the 32(kv) x 32(q) tile of kv chunk c
-  auto gemm_s = [&](const ACCT_LDS char* kbuf, f32x16 (&s)[QG][KT]) {
+  auto gemm_s = [&](const ACCT_LDS char* kbuf, int j, f32x16 (&s)[QG][KT]) {
+    if (BIAS && acc_bias) {
+      // element (c, r) belongs to key 32 c + 8 (r/4) + 4 g + r%4 of the tile, whatever the lane's row
 #pragma unroll
-    for (int gq = 0; gq < QG; gq++)
+      for (int gq = 0; gq < QG; gq++)
 #pragma unroll
-      for (int c = 0; c < KT; c++)
+        for (int c = 0; c < KT; c++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) s[gq][c][r] = 0.f;
+          for (int r4 = 0; r4 < 4; r4++) {
+            const typename E::V4 bv = bias_tile_read<T>(bias_lds + gq * 4096 + (j & 1) * 256, 0, 4 * c + r4, g);
+#pragma unroll
+            for (int e = 0; e < 4; e++) s[gq][c][4 * r4 + e] = (float)bv[e] * a.inv_scale;
+          }
+    } else {
+#pragma unroll
+      for (int gq = 0; gq < QG; gq++)
+#pragma unroll
+        for (int c = 0; c < KT; c++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) s[gq][c][r] = 0.f;
+    }
     // K fragments travel through a ring of FRING register sets: FRING reads are in flight ahead of the
     // MFMA that consumes the oldest one, so that a wave covers the LDS latency (well over one MFMA) by
     // itself.  The scheduling barriers keep the compiler from folding the ring back into read-wait-MFMA.
@@ -231,7 +255,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
     for (int gq = 0; gq < QG; gq++) {
       const int qrow = wq0 + 32 * gq + l32;
       const int qrow_c = min(qrow, a.Sq - 1);            // clamped for side-input addressing
-      if (BIAS) {
+      if (BIAS && !acc_bias) {
         if (bias_staged) {
           typename E::V4 bv[2][4];
 #pragma unroll
@@ -369,15 +393,16 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
         stage_tile(kdma, kp, a.k_ss, j + 1, nb);
         stage_tile(vdma, vp, a.v_ss, j + 1, nb + TILEB);
         DropStage::issue(a, bh, wq0, j + 1, lane, drop_lds + (buf ^ 1) * DropStage::BYTES);
+        if (BIAS && acc_bias && wq0 < a.Sq) stage_bias(j + 1);
       }
       const uint32_t info = classify(j);
       if (info & kAct) {
         f32x16 s[QG][KT];
         V8 pf[QG][KT][2];
-        gemm_s(kbuf, s);
+        gemm_s(kbuf, j, s);
         softmax(j, buf, info, s, pf);
         gemm_pv(vbuf, pf);
-      } else if (BIAS && bias_staged && j < j_hi && wq0 < a.Sq) {
+      } else if (BIAS && bias_staged && !acc_bias && j < j_hi && wq0 < a.Sq) {
         stage_bias(j + 1);                                  // nothing to read in this step: the region is free
       }
       dma_wait();
@@ -389,7 +414,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   // LDS region (pitch 2D+16 keeps the 8-byte writes of 16 rows on distinct banks) so that the
   // global stores are whole rows. ----
   T* op = (T*)a.o + b * a.o_sb + h * a.o_sh;
-  const float mnat = BIAS ? 1.0f : a.scale;
+  const float mnat = scaled ? 1.0f : a.scale;
   constexpr int OPITCH = C::DB * 64 + 16;
   ACCT_LDS char* obuf = smem + wave * (32 * OPITCH);
 #pragma unroll
@@ -424,17 +449,15 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
 }
 
 
-template <typename T, int D, int QG, int NW, bool BIAS, bool DROP>
-static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
+template <typename T, int D, int QG, int NW, bool BIAS, bool DROP, int KT>
+static hipError_t launch_fwd_kt(FaArgs a, hipStream_t st) {
   using C = SwzCfg<D>;
   constexpr int BM = 32 * QG * NW;
   a.n_tiles = (a.Sq + BM - 1) / BM;
   const bool mask_t = BIAS || DROP || a.mask_kind == kMaskDense || a.mask_kind == kMaskTile;
-  // The variants without a bias stream K/V in tiles of 128 keys where registers and LDS allow
-  // (8 waves x 32 rows, D <= 128): twice the matrix work between two barriers, -2 % (causal) to -6 % (full).
-  constexpr bool BIG = !BIAS && QG == 1 && NW == 8 && D <= 128;
-  constexpr int KT = BIG ? 4 : 2;
-  const size_t tiles = 4 * 32 * KT * (size_t)C::PITCH + (BIAS ? (size_t)NW * QG * 4096 : 0) + (size_t)NW * 2 * DropRowStage<DROP, QG, KT>::BYTES, stage = (size_t)NW * 32 * (C::DB * 64 + 16);
+  constexpr size_t biasb = BIAS ? (KT == 4 ? 512 : QG * 4096) : 0;     // per wave, as in the kernel
+  const size_t tiles = 4 * 32 * KT * (size_t)C::PITCH + NW * biasb + (size_t)NW * 2 * DropRowStage<DROP, QG, KT>::BYTES, stage = (size_t)NW * 32 * (C::DB * 64 + 16);
+  static_assert(4 * 32 * KT * (size_t)C::PITCH + NW * biasb + (size_t)NW * 2 * DropRowStage<DROP, QG, KT>::BYTES <= 160 * 1024, "the workgroup's LDS must fit the CU's 160 KB");
   const size_t smem = tiles > stage ? tiles : stage;
   auto kern = mask_t ? fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, true, KT> : fa_fwd_kernel<T, D, QG, NW, BIAS, DROP, BIAS || DROP, KT>;
   hipError_t e = allow_dynamic_lds((const void*)kern, smem);
@@ -442,6 +465,20 @@ static hipError_t launch_fwd_t(FaArgs a, hipStream_t st) {
   const long long nblk = (long long)a.n_tiles * a.B * a.N;
   hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(64 * NW), smem, st, a);
   return hipGetLastError();
+}
+
+template <typename T, int D, int QG, int NW, bool BIAS, bool DROP>
+static hipError_t launch_fwd_t(const FaArgs& a, hipStream_t st) {
+  // K/V stream in tiles of 128 keys where registers and LDS allow (8 waves x 32 rows, D <= 128): twice the
+  // matrix work between two barriers, -2 % (causal) to -6 % (full).  A bias tile per wave does not fit beside
+  // them; a key-only bias that the DMA can stage (the kernel's own test, repeated here) is a 256-byte row and does.
+  constexpr bool BIG = QG == 1 && NW == 8 && D <= 128;
+  if constexpr (BIG && BIAS) {
+    const bool row_staged = a.al_sq == 0 && (a.Sk & 7) == 0 && (((uintptr_t)a.alibi & 15) | ((a.al_sb | a.al_sh) & 7)) == 0;
+    return row_staged ? launch_fwd_kt<T, D, QG, NW, BIAS, DROP, 4>(a, st) : launch_fwd_kt<T, D, QG, NW, BIAS, DROP, 2>(a, st);
+  } else {
+    return launch_fwd_kt<T, D, QG, NW, BIAS, DROP, BIG ? 4 : 2>(a, st);
+  }
 }
 
 // SIDE = false: the head dims of the inference operator, built without the bias and dropout variants

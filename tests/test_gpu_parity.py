@@ -1095,6 +1095,30 @@ def test_full_size_alibi():
                    (o[sl], lse[sl], tuple(t[sl] for t in g)))
 
 
+@pytest.mark.parametrize("dtype, D", [(torch.float16, 128), (torch.bfloat16, 64), (torch.float16, 80)])
+def test_key_only_bias_on_the_eight_wave_forward(dtype, D):
+    # enough workgroups for the 8-wave forward, which streams 128-key tiles and takes a key-only bias as the
+    # initial value of its score accumulators; with key padding and dropout on top
+    B, N, S = 4, 16, 1024
+    q, k, v, dO = (_gen((B, N, S, D), 1201 + s, dtype) for s in range(4))
+    al = (0.5 * torch.randn((B, N, 1, S), generator=torch.Generator().manual_seed(1205))).to(dtype)
+    rng = np.random.default_rng(1206)
+    lens = np.array([1024, 700, 333, 900])
+    mask = (np.arange(S)[None, None, :] >= lens[:, None, None]).astype(np.uint8) | np.triu(np.ones((1, S, S), np.uint8), 1)
+    drop = (rng.random((B, N, S, S)) < 0.9).astype(np.uint8)
+    scale = D ** -0.5
+    tol = dict(atol=ATOL_BF16, rtol=RTOL_BF16) if dtype == torch.bfloat16 else {}
+    for with_drop in (False, True):
+        kw = dict(drop_mask=drop, keep_prob=0.9) if with_drop else {}
+        o, lse, g = _run(q, k, v, dO, scale=scale, mask_kind=_capi.MASK_DENSE_U8, attn_mask=mask, alibi=al, **kw)
+        for b, h in _sample_heads(B, N, n=3, seed=7):
+            sl = (slice(b, b + 1), slice(h, h + 1))
+            okw = dict(scale=scale, attn_mask=mask[b:b + 1], alibi=al[sl].float().numpy())
+            if with_drop:
+                okw.update(drop_mask=drop[sl], keep_prob=0.9)
+            _check_all(q[sl], k[sl], v[sl], dO[sl], okw, (o[sl], lse[sl], tuple(t[sl] for t in g)), **tol)
+
+
 def test_full_size_triangle_block_skip():
     # B=8, N=32, S=4096, D=128 forward, 128x128 blocks: block-skip vs the full-mask path
     B, N, S, D = 8, 32, 4096, 128
