@@ -232,8 +232,10 @@ def fa_fwd(p, q):
     return o, lse
 
 
-def fa_bwd(p, q, k, v, o, do, lse):
-    """Run acct_fa_bwd; returns (dQ, dK, dV) laid out like q, k, v."""
+def fa_bwd(p, q, k, v, o, do, lse, workspace_bytes=None):
+    """Run acct_fa_bwd; returns (dQ, dK, dV) laid out like q, k, v.  `workspace_bytes`: the size of the
+    workspace to pass instead of acct_fa_bwd_workspace_bytes (a smaller one that still holds the required
+    parts makes the library run the dK/dV kernel without splitting the query range)."""
     lib = load()
     if not q.is_cuda:
         raise RuntimeError("acct_fa_bwd needs device tensors (there is no CPU path)")
@@ -246,7 +248,7 @@ def fa_bwd(p, q, k, v, o, do, lse):
     dq = torch.empty_strided(q.size(), q.stride(), dtype=q.dtype, device=q.device)
     dk = torch.empty_strided(k.size(), k.stride(), dtype=k.dtype, device=k.device)
     dv = torch.empty_strided(v.size(), v.stride(), dtype=v.dtype, device=v.device)
-    nws = lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p))
+    nws = lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p)) if workspace_bytes is None else int(workspace_bytes)
     ws = _workspace(nws, q.device)
     with torch.cuda.device(q.device):
         _check(lib.acct_fa_bwd(ctypes.byref(p), _ptr(o), _ptr(do), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv),

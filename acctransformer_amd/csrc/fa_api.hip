@@ -235,11 +235,18 @@ size_t acct_fa_drop_bits_bytes(const acct_fa_params* p) {
   return droprow_bytes(p) + dropcol_bytes(p);
 }
 
-size_t acct_fa_bwd_workspace_bytes(const acct_fa_params* p) {
-  if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0) return 0;
-  if (p->Sk <= 0) return 0;
+// what the backward cannot do without: D and the exp2 offsets, the mask classes and bitmaps, the keep bits
+static size_t bwd_min_workspace_bytes(const acct_fa_params* p) {
   return 2 * align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + flag_bytes(p) + colbit_bytes(p) +
          (p->drop_bits ? 0 : droprow_bytes(p) + dropcol_bytes(p));
+}
+
+size_t acct_fa_bwd_workspace_bytes(const acct_fa_params* p) {
+  if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0) return 0;
+  if (p->Sk <= 0 || p->D <= 0) return 0;
+  // plus room for the per-slice sums of a dK/dV launch that splits the query range (few heads, short key
+  // sequence); a caller that passes less gets the unsplit launch
+  return align_up(bwd_min_workspace_bytes(p), 256) + acct::dkdv_split(p->B, p->N, p->Sq, p->Sk, p->D).part_bytes;
 }
 
 int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, size_t workspace_bytes, void* stream) {
@@ -293,9 +300,10 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
   if (((uintptr_t)O | (uintptr_t)dO | (uintptr_t)dQ | (uintptr_t)dK | (uintptr_t)dV) & 15)
     return fail(ACCT_E_SHAPE, "O, dO, dQ, dK and dV must be 16-byte aligned");
   if (p->keep_prob < 1.f && !dropout_on(p)) return fail(ACCT_E_NULLPTR, "keep_prob < 1 needs a drop_mask or drop_philox");
-  const size_t need = acct_fa_bwd_workspace_bytes(p);
+  const size_t need = bwd_min_workspace_bytes(p);
   if (!workspace || workspace_bytes < need)
-    return fail(ACCT_E_WORKSPACE, "backward workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
+    return fail(ACCT_E_WORKSPACE, "backward workspace too small: need %zu bytes (%zu to let the dK/dV kernel split the query range), got %zu",
+                need, acct_fa_bwd_workspace_bytes(p), workspace_bytes);
   if ((uintptr_t)workspace & 255) return fail(ACCT_E_WORKSPACE, "workspace must be 256-byte aligned");
   int n_cu = 0;
   rc = check_device(&n_cu);
@@ -339,6 +347,15 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
       if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "dropout bitmap kernel: %s", hipGetErrorString(e));
     }
   }
+  a.q_split = 1;
+  if (want_dkdv) {
+    const acct::DkdvSplit sp = acct::dkdv_split(p->B, p->N, p->Sq, p->Sk, p->D);
+    const size_t part_at = align_up(need, 256);
+    if (sp.q_split > 1 && workspace_bytes >= part_at + sp.part_bytes) {
+      a.q_split = sp.q_split;
+      a.dkdv_part = (float*)((char*)workspace + part_at);
+    }
+  }
   hipError_t e = acct::launch_bwd(a, p->dtype, p->D, stages, st);
   if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "backward kernels: %s", hipGetErrorString(e));
   return ACCT_OK;
@@ -354,7 +371,7 @@ int acct_fa_bwd_static(const acct_fa_params* p, const void* O, const void* dO, c
   g_err[0] = 0;
   int rc = validate(p, true);
   if (rc) return rc;
-  const size_t need = acct_fa_bwd_workspace_bytes(p);
+  const size_t need = bwd_min_workspace_bytes(p);
   if (need > (size_t)ACCT_FA_STATIC_SCRATCH_BYTES)
     return fail(ACCT_E_WORKSPACE, "acct_fa_bwd_static: this problem needs %zu bytes of scratch, the built-in buffer holds %zu; "
                 "use acct_fa_bwd with a caller-owned workspace", need, (size_t)ACCT_FA_STATIC_SCRATCH_BYTES);

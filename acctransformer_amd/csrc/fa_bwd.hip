@@ -419,6 +419,84 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   }
 }
 
+// Epilogue of the dK/dV kernel: dV (V role) or dK (K role) of a wave's key rows, scaled, converted and transposed
+// through the wave's own LDS region so that the global stores are whole rows.  acc[gk][db] = [d rows of block db,
+// key column l32] of key group gk; wk0 = first key row of the wave's pair.
+template <typename T, int D, int NGK>
+ACCT_DEV void dkdv_store_rows(const f32x16 (&acc)[NGK][SwzCfg<D>::DB], const FaArgs& a, int b, int h, int wk0, bool krole,
+                              float oscale, ACCT_LDS char* smem) {
+  using E = Elem<T>;
+  using C = SwzCfg<D>;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, g = lane >> 5;
+  T* outp = krole ? (T*)a.dk + b * a.k_sb + h * a.k_sh : (T*)a.dv + b * a.v_sb + h * a.v_sh;
+  const int64_t oss = krole ? a.k_ss : a.v_ss;
+  constexpr int OPITCH = C::DB * 64 + 16;
+  ACCT_LDS char* obuf = smem + wave * (32 * OPITCH);
+#pragma unroll
+  for (int gk = 0; gk < NGK; gk++) {
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; r4++) {
+        typename E::V2 t0 = E::cvt2(acc[gk][db][4 * r4 + 0] * oscale, acc[gk][db][4 * r4 + 1] * oscale);
+        typename E::V2 t1 = E::cvt2(acc[gk][db][4 * r4 + 2] * oscale, acc[gk][db][4 * r4 + 3] * oscale);
+        typename E::V4 ov = {t0[0], t0[1], t1[0], t1[1]};
+        *reinterpret_cast<ACCT_LDS typename E::V4*>(obuf + l32 * OPITCH + (32 * db + 8 * r4 + 4 * g) * 2) = ov;
+      }
+    const int nch = a.hd >> 3;                       // valid 16-byte chunks per row
+    const uint32_t nch_inv = recip16(nch);
+#pragma unroll
+    for (int i = 0; i < (32 * C::CPR + 63) / 64; i++) {
+      const int idx = lane + 64 * i;
+      const int r = div_small(idx, nch_inv), ch = idx - r * nch;
+      const int grow = wk0 + 32 * gk + r;
+      if (idx < 32 * nch && grow < a.Sk) {
+        const u32x4 v = *reinterpret_cast<const ACCT_LDS u32x4*>(obuf + r * OPITCH + ch * 16);
+        *reinterpret_cast<u32x4*>(outp + (int64_t)grow * oss + ch * 8) = v;
+      }
+    }
+  }
+}
+
+// Second half of a dK/dV launch whose query range was cut into a.q_split slices (few heads and a short key
+// sequence would otherwise leave most of the chip idle): one workgroup per key tile, the same wave and lane
+// roles as the dK/dV kernel; every lane adds up its accumulators over the slices in ascending order (a fixed
+// order: the result does not depend on which slice finished first) and stores the rows.
+template <typename T, int D, int NGK>
+__global__ void __launch_bounds__(512) fa_bwd_dkdv_reduce_kernel(const FaArgs a, float drop_scale) {
+  using C = SwzCfg<D>;
+  constexpr int NW = 8, WK = 32 * NGK, BNK = 4 * WK;
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const bool krole = wave >= 4;
+  const int BH = a.B * a.N, n_wg = BH * a.n_tiles, wg = blockIdx.x;
+  int bh, kt;
+  wg_map(wg, BH, a.n_tiles, bh, kt);
+  const int b = bh / a.N, h = bh % a.N;
+  const int wk0 = kt * BNK + (wave & 3) * WK;
+  f32x16 acc[NGK][C::DB];
+#pragma unroll
+  for (int gk = 0; gk < NGK; gk++)
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[gk][db][r] = 0.f;
+  for (int slice = 0; slice < a.q_split; slice++) {
+    const float* part = a.dkdv_part + ((((int64_t)slice * n_wg + wg) * NW + wave) * (NGK * C::DB) << 10) + lane * 16;
+#pragma unroll
+    for (int gk = 0; gk < NGK; gk++)
+#pragma unroll
+      for (int db = 0; db < C::DB; db++) {
+        const f32x16 v = *reinterpret_cast<const f32x16*>(part + ((gk * C::DB + db) << 10));
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[gk][db][r] += v[r];
+      }
+  }
+  const float oscale = (krole ? a.scale : drop_scale) * a.p_unshift;
+  dkdv_store_rows<T, D, NGK>(acc, a, b, h, wk0, krole, oscale, smem);
+}
+
 // ============================================================================
 // dK/dV kernel: kv-tile owner, 8 waves in 4 pairs.  A pair owns 64 key rows.
 // Its first wave (V role) keeps the K fragments of those rows in registers,
@@ -460,9 +538,14 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, g = lane >> 5;
   const int pair = __builtin_amdgcn_readfirstlane(wave & 3);   // wave-uniform: the pair's key range stays in scalar registers
   const bool krole = wave >= 4;                     // false: V role (S, P, dV); true: K role (dP, dS, dK)
-  const int BH = a.B * a.N;
+  const int BH = a.B * a.N, n_wg = BH * a.n_tiles;
+  int wg = blockIdx.x, slice = 0;                   // q_split > 1: the grid holds every key tile once per query slice
+  if (a.q_split > 1) {
+    slice = wg / n_wg;
+    wg -= slice * n_wg;
+  }
   int bh, kt;                                       // causal: the first key tiles are the heaviest
-  wg_map(blockIdx.x, BH, a.n_tiles, bh, kt);
+  wg_map(wg, BH, a.n_tiles, bh, kt);
   const int b = bh / a.N, h = bh % a.N;
   const int k0 = kt * BNK;
   const int wk0 = k0 + pair * WK;                   // first key row of this pair
@@ -478,6 +561,11 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   int i_lo = qb_lo * 2, i_hi = min(qb_hi * 2 + 1, (a.Sq - 1) / 64);
   const bool causal = a.mask_kind == kMaskCausal;
   if (causal) i_lo = max(i_lo, k0 / 64);            // query tiles wholly above the diagonal contribute 0
+  if (a.q_split > 1) {                              // this workgroup's slice of the 64-row query tiles
+    const int per = ((a.Sq + 63) / 64 + a.q_split - 1) / a.q_split;
+    i_lo = max(i_lo, slice * per);
+    i_hi = min(i_hi, (slice + 1) * per - 1);
+  }
   if (MASKT && a.mask_kind == kMaskDense) {
     // query tiles at either end whose blocks are wholly masked for every key block of this workgroup are
     // not streamed at all (key padding: a workgroup of padded keys has nothing to do)
@@ -846,36 +934,18 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     }
   }
 
-  // ---- epilogue: dV (V role) / scale * dK (K role), transposed through the wave's own LDS region ----
-  T* outp = krole ? (T*)a.dk + b * a.k_sb + h * a.k_sh : (T*)a.dv + b * a.v_sb + h * a.v_sh;
-  const int64_t oss = krole ? a.k_ss : a.v_ss;
-  const float oscale = (krole ? a.scale : (DROP ? a.inv_keep : 1.0f)) * a.p_unshift;
-  constexpr int OPITCH = C::DB * 64 + 16;
-  ACCT_LDS char* obuf = smem + wave * (32 * OPITCH);
+  if (a.q_split > 1) {
+    // this workgroup saw one slice of the query range: its sums go to the workspace as they sit in the registers
+    // (fa_bwd_dkdv_reduce_kernel adds the slices up in a fixed order and stores the rows)
+    float* part = a.dkdv_part + ((((int64_t)slice * n_wg + wg) * NW + wave) * (NGK * C::DB) << 10) + lane * 16;
 #pragma unroll
-  for (int gk = 0; gk < NGK; gk++) {
+    for (int gk = 0; gk < NGK; gk++)
 #pragma unroll
-    for (int db = 0; db < C::DB; db++)
-#pragma unroll
-      for (int r4 = 0; r4 < 4; r4++) {
-        typename E::V2 t0 = E::cvt2(acc[gk][db][4 * r4 + 0] * oscale, acc[gk][db][4 * r4 + 1] * oscale);
-        typename E::V2 t1 = E::cvt2(acc[gk][db][4 * r4 + 2] * oscale, acc[gk][db][4 * r4 + 3] * oscale);
-        typename E::V4 ov = {t0[0], t0[1], t1[0], t1[1]};
-        *reinterpret_cast<ACCT_LDS typename E::V4*>(obuf + l32 * OPITCH + (32 * db + 8 * r4 + 4 * g) * 2) = ov;
-      }
-    const int nch = a.hd >> 3;                       // valid 16-byte chunks per row
-    const uint32_t nch_inv = recip16(nch);
-#pragma unroll
-    for (int i = 0; i < (32 * C::CPR + 63) / 64; i++) {
-      const int idx = lane + 64 * i;
-      const int r = div_small(idx, nch_inv), ch = idx - r * nch;
-      const int grow = wk0 + 32 * gk + r;
-      if (idx < 32 * nch && grow < a.Sk) {
-        const u32x4 v = *reinterpret_cast<const ACCT_LDS u32x4*>(obuf + r * OPITCH + ch * 16);
-        *reinterpret_cast<u32x4*>(outp + (int64_t)grow * oss + ch * 8) = v;
-      }
-    }
+      for (int db = 0; db < C::DB; db++) *reinterpret_cast<f32x16*>(part + ((gk * C::DB + db) << 10)) = acc[gk][db];
+    return;
   }
+  const float oscale = (krole ? a.scale : (DROP ? a.inv_keep : 1.0f)) * a.p_unshift;
+  dkdv_store_rows<T, D, NGK>(acc, a, b, h, wk0, krole, oscale, smem);
 }
 
 #undef FOFF
@@ -913,8 +983,16 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
     auto kern = mask_t ? fa_bwd_dkdv_kernel<T, D, BIAS, DROP, true, NGK> : fa_bwd_dkdv_kernel<T, D, BIAS, DROP, BIAS || DROP, NGK>;
     e = allow_dynamic_lds((const void*)kern, smem2);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((unsigned)((long long)a.n_tiles * a.B * a.N)), dim3(512), smem2, st, a);
+    const long long n_wg = (long long)a.n_tiles * a.B * a.N;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(n_wg * (a.q_split > 1 ? a.q_split : 1))), dim3(512), smem2, st, a);
     e = hipGetLastError();
+    if (e == hipSuccess && a.q_split > 1) {
+      auto red = fa_bwd_dkdv_reduce_kernel<T, D, NGK>;
+      e = allow_dynamic_lds((const void*)red, epib);
+      if (e != hipSuccess) return e;
+      hipLaunchKernelGGL(red, dim3((unsigned)n_wg), dim3(512), epib, st, a, DROP ? a.inv_keep : 1.0f);
+      e = hipGetLastError();
+    }
   }
   return e;
 }

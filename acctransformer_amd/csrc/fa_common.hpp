@@ -105,6 +105,7 @@ struct FaArgs {
   void* o; float* lse;                 // fwd outputs / bwd inputs
   const void* dout; void* dq; void* dk; void* dv;                // bwd only
   float* delta; float* nlse;           // bwd workspace: D = rowsum(dO*O) and -LSE*log2(e), [B,N,Sq] each
+  float* dkdv_part;                    // q_split > 1: per-slice dK / dV sums of the dK/dV kernel, [q_split][workgroup][wave][regs x 64 lanes]
   const uint8_t* mask; const uint8_t* drop; const void* alibi;   // mask / drop: elements of mask_es / drop_es bytes
   const uint8_t* blkflags;             // [MB, Tr, Tc] block classes of a dense mask
   const uint32_t* droprow;             // [B*N*Sq, droprow_w] keep bits of the dropout mask by query row: bit k of word w = drop[row][32w+k] != 0
@@ -131,6 +132,7 @@ struct FaArgs {
   int mask_es, drop_es;                // bytes per element of mask and drop: 1 (uint8) or 2 (the I/O dtype); nonzero = masked / kept
   int row_prefix;                      // >0: row i sees keys j < (i/row_prefix + 1)*row_prefix only (multiple of 128)
   int n_tiles;                         // tiles along the owner dimension
+  int q_split;                         // dK/dV kernel: slices of the query range, each on workgroups of its own (1 = no split)
   int droprow_w;                       // 32-bit words per row of droprow: 2 * ceil(Sk / 64)
   uint32_t philox_k0, philox_k1;       // counter-based dropout: key, call offset and keep threshold (byte < thr keeps)
   uint32_t philox_offset, philox_thr;

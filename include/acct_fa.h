@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define ACCT_FA_VERSION 105
+#define ACCT_FA_VERSION 106
 
 /* error codes (0 = success) */
 #define ACCT_OK          0
@@ -147,6 +147,11 @@ size_t acct_fa_drop_bits_bytes(const acct_fa_params* p);
 int acct_fa_bwd(const acct_fa_params* p, const void* O, const void* dO, const float* LSE,
                 void* dQ, void* dK, void* dV,
                 void* workspace, size_t workspace_bytes, void* stream);
+/* Workspace of the backward, 256-byte aligned.  With few heads and a short key sequence (cross attention on 77
+ * keys: a handful of key tiles for 256 CUs) the size includes room for a dK/dV launch that cuts the query range
+ * into slices on workgroups of their own and adds the slices' sums in a second kernel (fixed order: still
+ * deterministic).  A smaller workspace that still holds everything else is accepted and runs the unsplit launch;
+ * the two launches differ in the last bits of dK and dV (another order of summation). */
 size_t acct_fa_bwd_workspace_bytes(const acct_fa_params* p);
 
 /* The two halves of acct_fa_bwd, for callers that need one side of the gradient
@@ -162,12 +167,12 @@ int acct_fa_bwd_dkdv(const acct_fa_params* p, const void* O, const void* dO, con
                      void* dK, void* dV, void* workspace, size_t workspace_bytes, void* stream);
 
 /* acct_fa_bwd for callers that cannot allocate or pass a workspace (code under HIP graph capture, serving loops,
- * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as acct_fa_bwd,
- * bit for bit, minus the workspace: D = rowsum(dO*O), the exp2 offsets, the mask block classes and bitmaps and
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments as acct_fa_bwd minus the
+ * workspace, and the results of acct_fa_bwd with a workspace of ACCT_FA_STATIC_SCRATCH_BYTES, bit for bit: D = rowsum(dO*O), the exp2 offsets, the mask block classes and bitmaps and
  * the dropout keep bits go to a buffer of ACCT_FA_STATIC_SCRATCH_BYTES that is part of the library's device
  * image (each GPU the library runs on holds one copy until the process ends).  The call allocates nothing and
- * frees nothing.  A problem whose acct_fa_bwd_workspace_bytes(p) exceeds the buffer is refused with
- * ACCT_E_WORKSPACE (pass drop_bits to keep a large dropout mask's bits out of it).  All calls on one GPU share
+ * frees nothing.  A problem that needs more than the buffer even without the optional split of the dK/dV launch
+ * is refused with ACCT_E_WORKSPACE (pass drop_bits to keep a large dropout mask's bits out of it).  All calls on one GPU share
  * the buffer: calls that may overlap on that GPU (different streams, different threads) race and must be
  * serialised by the caller; calls in one stream are ordered and safe.  Nothing in the buffer needs clearing
  * between calls: every region a call reads is written by that call first. */
