@@ -681,6 +681,51 @@ def test_wukong_training_shapes(D, Sq, Sk):
     _check_all(q, k, v, dO, dict(scale=D ** -0.5), (o, lse, (qd.grad, kd.grad, vd.grad)))
 
 
+@pytest.mark.parametrize("D, Sq, Sk, side", [(128, 2048, 300, "all"), (256, 1024, 256, "causal"), (80, 1536, 77, "bias"),
+                                             (64, 1100, 1100, "causal")])
+def test_dkdv_query_split_against_oracle_and_unsplit_launch(D, Sq, Sk, side):
+    # few key tiles: with the full workspace the dK/dV launch cuts the query range into slices and a second
+    # kernel adds them up; with the minimum workspace it runs unsplit.  Both against the oracle, and dQ (which
+    # the split does not touch) bit-equal between the two
+    B, N = 1, 2
+    q, dO = _gen((B, N, Sq, D), 940), _gen((B, N, Sq, D), 943)
+    k, v = _gen((B, N, Sk, D), 941), _gen((B, N, Sk, D), 942)
+    scale = D ** -0.5
+    okw, kw = dict(scale=scale), dict(scale=scale)
+    rng = np.random.default_rng(944)
+    if side == "all":
+        mask = (rng.random((B, Sq, Sk)) < 0.3).astype(np.uint8)
+        mask[:, :, 0] = 0
+        drop = (rng.random((B, N, Sq, Sk)) < 0.85).astype(np.uint8)
+        al = (0.3 * torch.randn((1, N, 1, Sk), generator=torch.Generator().manual_seed(945))).half()
+        okw.update(attn_mask=mask, drop_mask=drop, keep_prob=0.85, alibi=al.float().numpy())
+        kw.update(mask_kind=_capi.MASK_DENSE_U8, attn_mask=mask, drop_mask=drop, keep_prob=0.85, alibi=al)
+    elif side == "causal":
+        okw.update(attn_mask=np.triu(np.ones((1, Sq, Sk), np.uint8), 1))
+        kw.update(mask_kind=_capi.MASK_CAUSAL)
+    else:
+        al = (0.3 * torch.randn((B, N, 1, Sk), generator=torch.Generator().manual_seed(946))).half()
+        okw.update(alibi=al.float().numpy())
+        kw.update(alibi=al)
+    dev = lambda t: (torch.from_numpy(t) if isinstance(t, np.ndarray) else t).to(DEV)
+    mk = {n: dev(x) for n, x in kw.items() if n in ("attn_mask", "drop_mask", "alibi")}
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    p = _capi.make_params(qd, kd, vd, **{**kw, **mk})
+    lib = _capi.load()
+    o, lse = _capi.fa_fwd(p, qd)
+    full = lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p))
+    g_split = _capi.fa_bwd(p, qd, kd, vd, o, dO.to(DEV), lse)
+    # the slices' sums are the last part of the workspace, well over 256 bytes: a workspace that is 256 bytes
+    # short cannot hold them, and the launch is not split
+    stats = 2 * ((B * N * Sq * 4 + 255) // 256 * 256)
+    assert full - stats >= (1 << 20), "this shape is expected to split its dK/dV launch"
+    g_plain = _capi.fa_bwd(p, qd, kd, vd, o, dO.to(DEV), lse, workspace_bytes=full - 256)
+    torch.cuda.synchronize()
+    assert torch.equal(g_split[0], g_plain[0])
+    _check_all(q, k, v, dO, okw, (o, lse, g_split))
+    _check_all(q, k, v, dO, okw, (o, lse, g_plain))
+
+
 def test_layer_dropout_state_can_be_fixed_by_the_caller():
     # a forward that is run again (activation checkpointing) must draw the same mask: dropout_state fixes the stream
     B, N, S, D = 1, 2, 256, 64
