@@ -412,6 +412,13 @@ ACCT_DEV typename Elem<T>::V4 bias_tile_read(const ACCT_LDS char* tile, int row,
   return *reinterpret_cast<const ACCT_LDS typename Elem<T>::V4*>(tile + row * 128 + ((cc ^ (row & 7)) << 4) + 8 * half);
 }
 
+// x = (k > v) ? y : x for a constant k, as one compare into VCC and one select.  Written in C++, a run of these
+// is compiled into a batch of compares whose results sit in scalar register pairs; dozens of them push the
+// kernel's other scalars into spill lanes.
+ACCT_DEV float select_if_gt(float x, int k, int v, float y) {
+  asm("v_cmp_gt_i32_e32 vcc, %2, %1\n\tv_cndmask_b32_e32 %0, %0, %3, vcc" : "+v"(x) : "v"(v), "i"(k), "v"(y) : "vcc");
+  return x;
+}
 // all of this wave's direct-to-LDS loads have landed
 ACCT_DEV void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 

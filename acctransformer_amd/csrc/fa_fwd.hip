@@ -310,11 +310,14 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
           // the result is the same bit for bit at a third of the vector instructions.
           int vis = a.Sk - 1 - kv0 - 4 * g;                  // last visible key, relative to this lane's first
           if (diag) vis = min(vis, qrow - kv0 - 4 * g);
+          // (compare and select through VCC: see select_if_gt)
+          const float ninf = -INFINITY;
 #pragma unroll
-          for (int c = 0; c < KT; c++)
+          for (int c = 0; c < KT; c++) {
+            const int visc = vis - 32 * c;
 #pragma unroll
-            for (int r = 0; r < 16; r++)
-              if (32 * c + 8 * (r >> 2) + (r & 3) > vis) s[gq][c][r] = -INFINITY;
+            for (int r = 0; r < 16; r++) s[gq][c][r] = select_if_gt(s[gq][c][r], 8 * (r >> 2) + (r & 3), visc, ninf);
+          }
         }
       }
       // ---- online softmax for query row qrow ----
