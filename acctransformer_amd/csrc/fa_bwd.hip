@@ -684,8 +684,15 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
   };
 
   if (i_lo <= i_hi) {
-    stage(i_lo, smem);
-    if (BIAS && bias_staged) stage_bias(2 * i_lo);
+    // The query tiles are walked from the last one down: with a causal mask the key tiles of a head start at
+    // different rows (their diagonals) but all END at the last row, so walking down keeps the workgroups of a head
+    // -- they run side by side on one XCD -- on the same Q / dO tile at the same time, and one fetch from memory
+    // serves them all.  (Walking up, they stay four tiles apart and the XCD's L2 holds the tiles in between only
+    // just.)  Position p of the walk is tile i_hi - p; the two 32-row chunks of a tile keep their order.
+    const int ntile = i_hi - i_lo + 1, npos = 2 * ntile;
+    auto chunk_at = [&](int pos) { return 2 * (i_hi - (pos >> 1)) + (pos & 1); };
+    stage(i_hi, smem);
+    if (BIAS && bias_staged) stage_bias(chunk_at(0));
     // A full wait the compiler can see: the stationary fragments loaded above are complete, so it places
     // no vmcnt wait inside the loop -- such a wait would also stall on the next tile's DMA.
     __builtin_amdgcn_s_waitcnt(0);
@@ -695,6 +702,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     // publishes it and accumulates dV; the K role picks up P of chunk n-1.  One barrier per step,
     // nothing is carried across it in registers.
     const int c_lo = 2 * i_lo, c_hi = 2 * i_hi + 1;
+    (void)c_lo;
     // offsets of the transposed fragments of d block db: kept across the steps where the registers allow
     // (a fifth of the step's vector instructions otherwise), re-derived in every step in the bias + dropout variant
     constexpr bool KEEP_TOFF = !(BIAS && DROP);
@@ -713,11 +721,12 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     }
     const uint8_t* flcol = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + (int64_t)mb * a.Tr * a.Tc + wkb : nullptr;
     BlkClassWindow flwin;
-    flwin.init(flcol, a.Tc, c_lo >> 2, c_hi >> 2, lane);
-    for (int n = c_lo; n <= c_hi + 1; n++) {
-      if ((n & 1) && (n >> 1) < i_hi) stage((n >> 1) + 1, smem + ((((n >> 1) + 1 - i_lo) & 1) * STAGEB));
-      const int cidx = __builtin_amdgcn_readfirstlane(krole ? n - 1 : n);   // the chunk this wave works on in this step (wave-uniform: scalar)
-      if (cidx >= c_lo && cidx <= c_hi) {
+    flwin.init_descending(flcol, a.Tc, c_lo >> 2, c_hi >> 2, lane);
+    for (int n = 0; n <= npos; n++) {
+      if ((n & 1) && (n >> 1) + 1 < ntile) stage(i_hi - ((n >> 1) + 1), smem + ((((n >> 1) + 1) & 1) * STAGEB));
+      const int cpos = __builtin_amdgcn_readfirstlane(krole ? n - 1 : n);   // position of the chunk this wave works on in this step (wave-uniform: scalar)
+      if (cpos >= 0 && cpos < npos) {
+        const int cidx = chunk_at(cpos);
         const uint32_t cls = classify(cidx, flwin.get(cidx >> 2, lane));
         const bool act = cls & 1u, apply_mask = cls & 2u, limits = cls & 4u, diag = cls & 8u;
         const bool edge = (BIAS && !bias_staged && !row_bias) || apply_mask || limits;   // (a staged or per-key bias is already inside the scores)
@@ -742,7 +751,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 #pragma unroll
             for (int db = 0; db < 2; db++) toff2[db] = trow * C::PITCH + swz_off(4 * db + tchunk, C::swz(trow)) + 8 * (ln & 1);
           }
-          ACCT_LDS char* qbuf = smem + (((cidx >> 1) - i_lo) & 1) * STAGEB;
+          ACCT_LDS char* qbuf = smem + ((cpos >> 1) & 1) * STAGEB;
           ACCT_LDS char* dobuf = qbuf + TILEB;
           const ACCT_LDS float* lbuf = (const ACCT_LDS float*)(qbuf + 2 * TILEB);
           const ACCT_LDS float* dbuf = lbuf + 64;
@@ -794,7 +803,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
           }
           if (BIAS && bias_staged) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // bias tile consumed: stage the next chunk's
-            if (n < c_hi) stage_bias(n + 1);
+            if (cpos + 1 < npos) stage_bias(chunk_at(cpos + 1));
           }
           uint32_t dcw[NGK] = {};                       // keep bits of the chunk's 32 rows for this lane's two key columns
           if (DROP) {
@@ -925,8 +934,8 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
               if (i + BRING < NT) tr[i % BRING] = tread(i + BRING);
             }
           }
-        } else if (BIAS && bias_staged && n < c_hi) {
-          stage_bias(n + 1);                            // nothing to read in this step: the region is free
+        } else if (BIAS && bias_staged && cpos + 1 < npos) {
+          stage_bias(chunk_at(cpos + 1));               // nothing to read in this step: the region is free
         }
       }
       dma_wait();                                     // a tile requested at the top of this step has landed

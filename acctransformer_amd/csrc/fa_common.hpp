@@ -182,15 +182,20 @@ ACCT_DEV void trim_dead_tiles(int& lo, int& hi, int lane, F dead) {
 // masks in scalar registers: one byte load per lane and two ballots fill the window, and a step of the
 // tile loop then looks its block up with scalar shifts.  (A byte load per step would stall the step for
 // a round trip to memory, since the class decides a wave-uniform branch.)  Blocks are asked for in
-// ascending order; the window moves on when the block asked for lies past its end.
+// ascending order (init) or in descending order (init_descending); the window moves on when the block asked
+// for lies outside it.
 struct BlkClassWindow {
   const uint8_t* p;
   int64_t stride;
-  int last, base;
+  int first, last, base;
   uint64_t b0, b1;
-  ACCT_DEV void init(const uint8_t* p_, int64_t stride_, int first, int last_, int lane) {
-    p = p_; stride = stride_; last = last_;
+  ACCT_DEV void init(const uint8_t* p_, int64_t stride_, int first_, int last_, int lane) {
+    p = p_; stride = stride_; first = first_; last = last_;
     load(first, lane);
+  }
+  ACCT_DEV void init_descending(const uint8_t* p_, int64_t stride_, int first_, int last_, int lane) {
+    p = p_; stride = stride_; first = first_; last = last_;
+    load(max(first_, last_ - 63), lane);
   }
   ACCT_DEV void load(int first, int lane) {
     base = first;
@@ -201,6 +206,7 @@ struct BlkClassWindow {
   }
   ACCT_DEV uint32_t get(int blk, int lane) {
     if (blk - base >= 64) load(blk, lane);
+    else if (blk < base) load(max(first, blk - 63), lane);
     const int sh = blk - base;
     return (uint32_t)((b0 >> sh) & 1u) | ((uint32_t)((b1 >> sh) & 1u) << 1);
   }
