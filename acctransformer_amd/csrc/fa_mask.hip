@@ -196,29 +196,30 @@ hipError_t launch_mask_colbits(const FaArgs& a, const uint8_t* flags, uint32_t* 
 }
 
 // Dropout mask (uint8 {0,1}, or the reference's {0, 1/keep_prob} in the I/O dtype; nonzero = keep) packed into keep bits, by query row for the kernels whose lanes own
-// query rows (forward, dQ) and by key column for the dK/dV kernel.  One wave per (batch*head, 128 query
-// rows, 1024 keys): per row every lane loads the 16 bytes of keys 16*lane .. +15 (a kilobyte per wave
+// query rows (forward, dQ) and by key column for the dK/dV kernel.  One wave per (batch*head, 32 query
+// rows, 1024 keys) -- enough waves to keep the memory system busy --: per row every lane loads the 16 bytes of keys 16*lane .. +15 (a kilobyte per wave
 // instruction keeps enough bytes in flight) and turns them into 16 bits; lane pairs form the 32-bit row words.
 //   rowbits [B*N*Sq, 2*ceil(Sk/64)] 32-bit: bit k of word w = keep[row][32w + k];
 //   colbits [B*N, Tr, Sk, 4] 32-bit: bit r of the 128-bit entry = keep[128*qb + r][key].
 template <int ES>
 __global__ void __launch_bounds__(64) fa_drop_bits_kernel(const FaArgs a, uint32_t* rowbits, uint32_t* colbits) {
   const int nspan = (a.Sk + 1023) / 1024;
-  const int span = blockIdx.x % nspan, qb = (blockIdx.x / nspan) % a.Tr, bh = blockIdx.x / (nspan * a.Tr);
+  const int i = blockIdx.x & 3;                         // which 32 rows of the 128-row block: word i of the column entries
+  const int blk = blockIdx.x >> 2;
+  const int span = blk % nspan, qb = (blk / nspan) % a.Tr, bh = blk / (nspan * a.Tr);
   const int lane = threadIdx.x;
   const int kv = span * 1024 + 16 * lane;               // first of this lane's sixteen keys
   const bool vec = (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 15) == 0 && kv + 16 <= a.Sk;   // (16 elements: ES aligned 16-byte loads)
   const int widx = 32 * span + (lane >> 1);             // this lane pair's word within the row
   const bool writer = rowbits && (lane & 1) == 0 && widx < a.droprow_w;
-  uint32_t* rowout = rowbits + ((int64_t)bh * a.Sq + qb * 128) * a.droprow_w + widx;
-  const uint8_t* p = a.drop + (((int64_t)bh * a.Sq + qb * 128) * a.Sk + min(kv, max(a.Sk - 16, 0))) * ES;
+  uint32_t* rowout = rowbits + ((int64_t)bh * a.Sq + qb * 128 + 32 * i) * a.droprow_w + widx;
+  const uint8_t* p = a.drop + (((int64_t)bh * a.Sq + qb * 128 + 32 * i) * a.Sk + min(kv, max(a.Sk - 16, 0))) * ES;
   const int nrow = min(128, a.Sq - qb * 128);
-  uint32_t cw[16][4];                                   // per key: four words of 32 rows, most significant bit first
+  uint32_t cw[16];                                      // per key: the word of these 32 rows, most significant bit first
+  {
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-#pragma unroll
-    for (int e = 0; e < 16; e++) cw[e][i] = 0u;
-#pragma unroll 4
+    for (int e = 0; e < 16; e++) cw[e] = 0u;
+#pragma unroll 8
     for (int r = 0; r < 32; r++) {
       const int rr = 32 * i + r;
       uint32_t nz = 0;                                  // bit e: this lane's key e of the row is kept
@@ -247,7 +248,7 @@ __global__ void __launch_bounds__(64) fa_drop_bits_kernel(const FaArgs a, uint32
       p += (int64_t)a.Sk * ES;                          // per-lane pointer walks down the rows
       const uint32_t bits = nz;
 #pragma unroll
-      for (int e = 0; e < 16; e++) cw[e][i] = (cw[e][i] << 1) | ((nz >> e) & 1u);
+      for (int e = 0; e < 16; e++) cw[e] = (cw[e] << 1) | ((nz >> e) & 1u);
       uint32_t x = bits << (16 * (lane & 1));
       x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xf, 0xf, true);    // lane ^ 1
       if (writer && rr < nrow) *rowout = x;
@@ -257,32 +258,29 @@ __global__ void __launch_bounds__(64) fa_drop_bits_kernel(const FaArgs a, uint32
   if (colbits) {
 #pragma unroll
     for (int e = 0; e < 16; e++)
-      if (kv + e < a.Sk) {
-        u32x4 v = {__builtin_bitreverse32(cw[e][0]), __builtin_bitreverse32(cw[e][1]), __builtin_bitreverse32(cw[e][2]),
-                   __builtin_bitreverse32(cw[e][3])};
-        *reinterpret_cast<u32x4*>(colbits + (((int64_t)bh * a.Tr + qb) * a.Sk + kv + e) * 4) = v;
-      }
+      if (kv + e < a.Sk) colbits[(((int64_t)bh * a.Tr + qb) * a.Sk + kv + e) * 4 + i] = __builtin_bitreverse32(cw[e]);
   }
 }
 
 // The same bitmaps for counter-based dropout: nothing is read, the keep decisions come from Philox4x32-10.
 // One call yields the 16 bytes of one (query row, 32-key group M, half g): keys 32M + 8u + 4g + e for
 // u = 0..3, e = 0..3 -- the keys one lane of the attention kernels owns in a 32-key group, so a kernel
-// could also draw them in place.  One wave per (batch*head, 128 query rows, 1024 keys); lane 2L + g owns
+// could also draw them in place.  One wave per (batch*head, 32 query rows, 1024 keys); lane 2L + g owns
 // (M = 32*span + L, g), the lane pair forms the 32-bit row word of group M.
 __global__ void __launch_bounds__(64) fa_drop_philox_kernel(const FaArgs a, uint32_t* rowbits, uint32_t* colbits) {
   const int nspan = (a.Sk + 1023) / 1024;
-  const int span = blockIdx.x % nspan, qb = (blockIdx.x / nspan) % a.Tr, bh = blockIdx.x / (nspan * a.Tr);
+  const int i = blockIdx.x & 3;                         // which 32 rows of the 128-row block: word i of the column entries
+  const int blk = blockIdx.x >> 2;
+  const int span = blk % nspan, qb = (blk / nspan) % a.Tr, bh = blk / (nspan * a.Tr);
   const int lane = threadIdx.x, g = lane & 1;
   const int grp = 32 * span + (lane >> 1);              // 32-key group = word index within the row
   const bool writer = rowbits && g == 0 && grp < a.droprow_w;
-  uint32_t* rowout = rowbits + ((int64_t)bh * a.Sq + qb * 128) * a.droprow_w + grp;
+  uint32_t* rowout = rowbits + ((int64_t)bh * a.Sq + qb * 128 + 32 * i) * a.droprow_w + grp;
   const int nrow = min(128, a.Sq - qb * 128);
-  uint32_t cw[16][4];                                   // per key: four words of 32 rows, most significant bit first
+  uint32_t cw[16];                                      // per key: the word of these 32 rows, most significant bit first
+  {
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-#pragma unroll
-    for (int t = 0; t < 16; t++) cw[t][i] = 0u;
+    for (int t = 0; t < 16; t++) cw[t] = 0u;
 #pragma unroll 2
     for (int r = 0; r < 32; r++) {
       const int rr = 32 * i + r;
@@ -293,7 +291,7 @@ __global__ void __launch_bounds__(64) fa_drop_philox_kernel(const FaArgs a, uint
       for (int t = 0; t < 16; t++) {                    // t = 4u + e
         const uint32_t keep = ((v[t >> 2] >> (8 * (t & 3))) & 0xffu) < a.philox_thr ? 1u : 0u;
         bits |= keep << (8 * (t >> 2) + (t & 3));
-        cw[t][i] = (cw[t][i] << 1) | (rr < nrow ? keep : 0u);
+        cw[t] = (cw[t] << 1) | (rr < nrow ? keep : 0u);
       }
       uint32_t x = bits << (4 * g);
       x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xf, 0xf, true);    // lane ^ 1
@@ -305,23 +303,19 @@ __global__ void __launch_bounds__(64) fa_drop_philox_kernel(const FaArgs a, uint
 #pragma unroll
     for (int t = 0; t < 16; t++) {
       const int key = 32 * grp + 8 * (t >> 2) + 4 * g + (t & 3);
-      if (key < a.Sk) {
-        u32x4 v = {__builtin_bitreverse32(cw[t][0]), __builtin_bitreverse32(cw[t][1]), __builtin_bitreverse32(cw[t][2]),
-                   __builtin_bitreverse32(cw[t][3])};
-        *reinterpret_cast<u32x4*>(colbits + (((int64_t)bh * a.Tr + qb) * a.Sk + key) * 4) = v;
-      }
+      if (key < a.Sk) colbits[(((int64_t)bh * a.Tr + qb) * a.Sk + key) * 4 + i] = __builtin_bitreverse32(cw[t]);
     }
   }
 }
 
 hipError_t launch_drop_philox(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st) {
-  const long long nblk = (long long)a.B * a.N * a.Tr * ((a.Sk + 1023) / 1024);
+  const long long nblk = 4LL * a.B * a.N * a.Tr * ((a.Sk + 1023) / 1024);
   hipLaunchKernelGGL(fa_drop_philox_kernel, dim3((unsigned)nblk), dim3(64), 0, st, a, rowbits, colbits);
   return hipGetLastError();
 }
 
 hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st) {
-  const long long nblk = (long long)a.B * a.N * a.Tr * ((a.Sk + 1023) / 1024);
+  const long long nblk = 4LL * a.B * a.N * a.Tr * ((a.Sk + 1023) / 1024);
   if (a.drop_es == 2) hipLaunchKernelGGL(fa_drop_bits_kernel<2>, dim3((unsigned)nblk), dim3(64), 0, st, a, rowbits, colbits);
   else hipLaunchKernelGGL(fa_drop_bits_kernel<1>, dim3((unsigned)nblk), dim3(64), 0, st, a, rowbits, colbits);
   return hipGetLastError();
