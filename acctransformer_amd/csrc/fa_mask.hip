@@ -47,6 +47,7 @@ __global__ void __launch_bounds__(1024) fa_mask_blocks_vec_kernel(const FaArgs a
         const int kv = (base + i) * 128 + c0;
         if (kv < a.Sk) {                                // Sk % 16 == 0: a piece is entirely inside or outside
           bool has_zero = false, has_nonzero = false;
+          const bool on_diag = base + i == qb;          // the per-element pattern matters on the diagonal block only
           uint32_t nz = 0;                              // bit e: element e of this thread's 16 is nonzero
 #pragma unroll
           for (int h = 0; h < ES; h++) {
@@ -57,20 +58,22 @@ __global__ void __launch_bounds__(1024) fa_mask_blocks_vec_kernel(const FaArgs a
                 // a byte is zero iff (x - 0x01010101) & ~x & 0x80808080 has its top bit set
                 has_nonzero |= v[w] != 0;
                 has_zero |= ((v[w] - 0x01010101u) & ~v[w] & 0x80808080u) != 0;
+                if (on_diag) {
 #pragma unroll
-                for (int e = 0; e < 4; e++) nz |= (((v[w] >> (8 * e)) & 0xffu) != 0 ? 1u : 0u) << (4 * w + e);
+                  for (int e = 0; e < 4; e++) nz |= (((v[w] >> (8 * e)) & 0xffu) != 0 ? 1u : 0u) << (4 * w + e);
+                }
               } else {
                 // 2-byte floating-point elements: the sign of a zero does not count
                 const uint32_t lo16 = v[w] & 0x7fffu, hi16 = (v[w] >> 16) & 0x7fffu;
                 has_nonzero |= (lo16 | hi16) != 0;
                 has_zero |= lo16 == 0 || hi16 == 0;
-                nz |= ((lo16 != 0 ? 1u : 0u) | (hi16 != 0 ? 2u : 0u)) << (8 * h + 2 * w);
+                if (on_diag) nz |= ((lo16 != 0 ? 1u : 0u) | (hi16 != 0 ? 2u : 0u)) << (8 * h + 2 * w);
               }
             }
           }
           if (has_nonzero) bm |= 1ull << i;
           if (has_zero) bu |= 1ull << i;
-          if (base + i == qb) {
+          if (on_diag) {
 #pragma unroll
             for (int e = 0; e < 16; e++) tri_bad |= (((nz >> e) & 1u) != 0) != (c0 + e > (tid >> 3));
           }
