@@ -778,7 +778,8 @@ def test_random_configurations_against_oracle(block):
             m = (rng.random((B, Sq, Sk)) < 0.3).astype(np.uint8); m[:, :, 0] = 0
             kw.update(mask_kind=_capi.MASK_DENSE_U8, attn_mask=m); okw.update(attn_mask=m)
         elif c["mask"] == "dense_padding":
-            lens = rng.integers(1, Sk + 1, size=B)
+            # (at least 16 live keys per sequence, for the reason given in _random_case)
+            lens = rng.integers(16, Sk + 1, size=B)
             m = np.ascontiguousarray(np.broadcast_to((np.arange(Sk)[None, None, :] >= lens[:, None, None]), (B, Sq, Sk)), dtype=np.uint8)
             kw.update(mask_kind=_capi.MASK_DENSE_U8, attn_mask=m); okw.update(attn_mask=m)
         elif c["mask"] == "dense_causal_f16":
