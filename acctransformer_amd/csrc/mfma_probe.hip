@@ -11,6 +11,10 @@
 
 #include "../../include/acct_fa.h"
 
+// Shader-clock and wall-clock (100 MHz) ticks that wave 0 of workgroup 0 spent in the MFMA loop of the last launch:
+// their ratio is the shader clock while the matrix pipe runs flat out.
+__device__ unsigned long long acct_probe_ticks[2];
+
 // Target of a store that practically never executes (referenced from device code only).  External linkage: the
 // compiler must not conclude that nobody reads it and drop the loop that feeds the store.
 __device__ float acct_probe_sink[512];
@@ -42,6 +46,9 @@ __global__ void __launch_bounds__(512) mfma_rate_kernel(int iters) {
   for (int n = 0; n < 4; n++)
 #pragma unroll
     for (int r = 0; r < 16; r++) c[n][r] = 0.f;
+  const bool timed = blockIdx.x == 0 && threadIdx.x < 64;                  // wave-uniform
+  unsigned long long t0 = 0, r0 = 0;
+  if (timed) { t0 = __builtin_amdgcn_s_memtime(); r0 = __builtin_amdgcn_s_memrealtime(); }
   for (int it = 0; it < iters; it++) {
 #pragma unroll
     for (int n = 0; n < kMfmaPerIter; n++) c[n & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c[n & 3], 0, 0, 0);
@@ -50,15 +57,20 @@ __global__ void __launch_bounds__(512) mfma_rate_kernel(int iters) {
 #pragma unroll
   for (int n = 0; n < 4; n++)
 #pragma unroll
-    for (int e = 0; e < 16; e++) r += c[n][e];
+    for (int e = 0; e < 16; e++) r += c[n][e];                // (waits for the last MFMA)
   if (r == 123.456f) acct_probe_sink[threadIdx.x] = r;        // practically never true: keeps the loop alive without a store
+  if (timed) {
+    const unsigned long long t1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+    if (lane == 0) { acct_probe_ticks[0] = t1 - t0; acct_probe_ticks[1] = r1 - r0; }
+  }
 }
 
 }  // namespace
 
-extern "C" int acct_probe_mfma_rate(int varying_operands, double* tflops, void* stream) {
+static int probe_mfma(int varying_operands, double* tflops, double* shader_ghz, void* stream) {
   if (!tflops) return ACCT_E_NULLPTR;
   *tflops = 0.0;
+  if (shader_ghz) *shader_ghz = 0.0;
   int dev = 0, n_cu = 0;
   if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n_cu <= 0)
     return ACCT_E_LAUNCH;
@@ -86,5 +98,19 @@ extern "C" int acct_probe_mfma_rate(int varying_operands, double* tflops, void* 
   if (e != hipSuccess || !(ms > 0.f)) return ACCT_E_LAUNCH;
   const double flop = (double)kTimed * n_cu * 8.0 * kItersPerLaunch * kMfmaPerIter * (2.0 * 32 * 32 * 16);
   *tflops = flop / (ms * 1e-3) / 1e12;
+  if (shader_ghz) {
+    unsigned long long ticks[2] = {0, 0};
+    if (hipMemcpyFromSymbol(ticks, HIP_SYMBOL(acct_probe_ticks), sizeof(ticks)) != hipSuccess || ticks[1] == 0) return ACCT_E_LAUNCH;
+    *shader_ghz = (double)ticks[0] / ((double)ticks[1] * 10.0);            // the wall clock ticks every 10 ns
+  }
   return ACCT_OK;
+}
+
+extern "C" int acct_probe_mfma_rate(int varying_operands, double* tflops, void* stream) {
+  return probe_mfma(varying_operands, tflops, nullptr, stream);
+}
+
+extern "C" int acct_probe_mfma_clock(int varying_operands, double* tflops, double* shader_ghz, void* stream) {
+  if (!shader_ghz) return ACCT_E_NULLPTR;
+  return probe_mfma(varying_operands, tflops, shader_ghz, stream);
 }

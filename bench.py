@@ -324,12 +324,14 @@ def main():
     # operands toggle (the clock follows the power drawn); the benchmark's N(0,1) data is the varying case.
     mfma = None
     if not args.no_mfma_probe:
-        rates = {}
+        rates, clocks = {}, {}
         for key, varying in (("varying_operands", 1), ("constant_operands", 0)):
-            r = ctypes.c_double(0.0)
-            check(lib.acct_probe_mfma_rate(varying, ctypes.byref(r), st))
+            r, ghz = ctypes.c_double(0.0), ctypes.c_double(0.0)
+            check(lib.acct_probe_mfma_clock(varying, ctypes.byref(r), ctypes.byref(ghz), st))
             rates[key] = round(r.value, 1)
-        mfma = {"unit": "TFLOP/s", "instruction": "v_mfma_f32_32x32x16_f16", **rates,
+            clocks[key] = round(ghz.value, 3)
+        # (shader clock a wave saw inside the loop: an MFMA takes 32 clocks either way, the power drawn sets the clock)
+        mfma = {"unit": "TFLOP/s", "instruction": "v_mfma_f32_32x32x16_f16", **rates, "shader_clock_ghz": clocks,
                 "frac_of_nominal_peak": round(rates["varying_operands"] / PEAK_FP16_TFLOPS, 4),
                 "dominant_kernel_frac_of_sustained": round(achieved / rates["varying_operands"], 4)}
     out = {

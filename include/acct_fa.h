@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define ACCT_FA_VERSION 106
+#define ACCT_FA_VERSION 107
 
 /* error codes (0 = success) */
 #define ACCT_OK          0
@@ -211,6 +211,11 @@ int acct_build_is_complete(void);
  * rate, depends on how much the operands toggle).  Runs about 0.1 s of kernels on `stream` and waits for them.
  * bench.py reports both figures beside the attention kernels' roofline fraction. */
 int acct_probe_mfma_rate(int varying_operands, double* tflops, void* stream);
+
+/* The same run, which also reports the shader clock (GHz) that one wave saw while it ran: shader-clock ticks
+ * over wall-clock ticks across its MFMA loop.  An MFMA of this kind occupies the matrix pipe for 32 clocks whatever
+ * the operands; what the power drawn changes is this clock.  Measurement aid, no counterpart in the reference. */
+int acct_probe_mfma_clock(int varying_operands, double* tflops, double* shader_ghz, void* stream);
 
 #ifdef __cplusplus
 }

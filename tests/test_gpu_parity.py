@@ -1117,6 +1117,14 @@ def test_mfma_rate_probe_reports_a_plausible_ceiling():
     assert 500.0 < rates[0] <= 2516.6 * 1.02, rates
     assert rates[1] >= 0.95 * rates[0], rates
     assert lib.acct_probe_mfma_rate(1, None, st) == -1
+    # the variant that also reports the shader clock inside the loop: the rate is that of the chip's 1024 SIMDs
+    # retiring one 32x32x16 MFMA (32768 flop) per 32 clocks at that clock (less the gaps between the launches)
+    r, ghz = ctypes.c_double(0.0), ctypes.c_double(0.0)
+    assert lib.acct_probe_mfma_clock(1, ctypes.byref(r), ctypes.byref(ghz), st) == 0, lib.acct_last_error().decode()
+    assert 0.8 < ghz.value < 2.6, ghz.value
+    n_simd = 4 * torch.cuda.get_device_properties(0).multi_processor_count
+    assert abs(r.value - n_simd * 32768 / 32.0 * ghz.value * 1e-3) < 0.15 * r.value, (r.value, ghz.value)
+    assert lib.acct_probe_mfma_clock(1, ctypes.byref(r), None, st) == -1
 
 
 # ---- both branches of the workgroup map (more / not more than 64 batch*head pairs) -------------------
