@@ -96,8 +96,6 @@ def load():
     lib.acct_probe_mfma_rate.restype = ctypes.c_int
     lib.acct_probe_mfma_clock.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
     lib.acct_probe_mfma_clock.restype = ctypes.c_int
-    lib.acct_probe_shader_clock.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
-    lib.acct_probe_shader_clock.restype = ctypes.c_int
     lib.acct_version.argtypes = []
     lib.acct_version.restype = ctypes.c_int
     _lib = lib

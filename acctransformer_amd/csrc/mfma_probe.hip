@@ -65,17 +65,6 @@ __global__ void __launch_bounds__(512) mfma_rate_kernel(int iters) {
   }
 }
 
-// One wave watches both counters for about 10 us (a bounded number of polls): the clock the power management holds
-// at this moment, i.e. the one the kernels that ran just before on the stream were given (it moves over milliseconds).
-__global__ void __launch_bounds__(64) clock_sample_kernel() {
-  const unsigned long long t0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
-  unsigned long long r1 = r0;
-  for (int i = 0; i < (1 << 16) && r1 - r0 < 1000; i++) r1 = __builtin_amdgcn_s_memrealtime();
-  const unsigned long long t1 = __builtin_amdgcn_s_memtime();
-  r1 = __builtin_amdgcn_s_memrealtime();
-  if (threadIdx.x == 0) { acct_probe_ticks[0] = t1 - t0; acct_probe_ticks[1] = r1 - r0; }
-}
-
 }  // namespace
 
 static int probe_mfma(int varying_operands, double* tflops, double* shader_ghz, void* stream) {
@@ -124,17 +113,4 @@ extern "C" int acct_probe_mfma_rate(int varying_operands, double* tflops, void* 
 extern "C" int acct_probe_mfma_clock(int varying_operands, double* tflops, double* shader_ghz, void* stream) {
   if (!shader_ghz) return ACCT_E_NULLPTR;
   return probe_mfma(varying_operands, tflops, shader_ghz, stream);
-}
-
-extern "C" int acct_probe_shader_clock(double* shader_ghz, void* stream) {
-  if (!shader_ghz) return ACCT_E_NULLPTR;
-  *shader_ghz = 0.0;
-  hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(clock_sample_kernel, dim3(1), dim3(64), 0, st);
-  unsigned long long ticks[2] = {0, 0};
-  if (hipGetLastError() != hipSuccess || hipStreamSynchronize(st) != hipSuccess ||
-      hipMemcpyFromSymbol(ticks, HIP_SYMBOL(acct_probe_ticks), sizeof(ticks)) != hipSuccess || ticks[1] == 0)
-    return ACCT_E_LAUNCH;
-  *shader_ghz = (double)ticks[0] / ((double)ticks[1] * 10.0);
-  return ACCT_OK;
 }

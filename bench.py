@@ -168,14 +168,6 @@ def main():
     t_dq = sum(e[1].elapsed_time(e[2]) for e in ev) / K
     t_dkdv = sum(e[2].elapsed_time(e[3]) for e in ev) / K
 
-    # the shader clock these kernels are given: sampled on the stream right behind another 50 untimed steps (the
-    # power management moves it over milliseconds; an idle GPU would read the boost clock)
-    for _ in range(50):
-        step(p)
-    ghz = ctypes.c_double(0.0)
-    check(lib.acct_probe_shader_clock(ctypes.byref(ghz), st))
-    step_clock_ghz = round(ghz.value, 3)
-
     # dense-mask reading of the same workload (untimed for `value`)
     ms_dense = None
     if not args.no_dense_pass:
@@ -356,7 +348,6 @@ def main():
         "triangle_block_skip": tri,
         "other_configs": other,
         "clock_settle": {"seconds": round(settle_s, 3), "steps": settle_steps},
-        "shader_clock_ghz_behind_the_steps": step_clock_ghz,
         "mfma_sustained": mfma,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": traffic_bytes[dom]},

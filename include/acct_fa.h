@@ -217,11 +217,6 @@ int acct_probe_mfma_rate(int varying_operands, double* tflops, void* stream);
  * the operands; what the power drawn changes is this clock.  Measurement aid, no counterpart in the reference. */
 int acct_probe_mfma_clock(int varying_operands, double* tflops, double* shader_ghz, void* stream);
 
-/* The shader clock (GHz) right now: one wave compares the two counters for about 10 us on `stream`, after whatever was
- * queued there before.  The power management moves the clock over milliseconds, so a call placed behind a long
- * run of kernels reads the clock those kernels were given.  Measurement aid, no counterpart in the reference. */
-int acct_probe_shader_clock(double* shader_ghz, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -1125,10 +1125,6 @@ def test_mfma_rate_probe_reports_a_plausible_ceiling():
     n_simd = 4 * torch.cuda.get_device_properties(0).multi_processor_count
     assert abs(r.value - n_simd * 32768 / 32.0 * ghz.value * 1e-3) < 0.15 * r.value, (r.value, ghz.value)
     assert lib.acct_probe_mfma_clock(1, ctypes.byref(r), None, st) == -1
-    # the plain clock sample
-    assert lib.acct_probe_shader_clock(ctypes.byref(ghz), st) == 0, lib.acct_last_error().decode()
-    assert 0.05 < ghz.value < 2.6, ghz.value
-    assert lib.acct_probe_shader_clock(None, st) == -1
 
 
 # ---- both branches of the workgroup map (more / not more than 64 batch*head pairs) -------------------
