@@ -42,6 +42,7 @@ class AcctFaParams(ctypes.Structure):
         ("attn_mask", ctypes.c_void_p), ("drop_mask", ctypes.c_void_p), ("alibi", ctypes.c_void_p),
         ("drop_seed", ctypes.c_uint64), ("drop_offset", ctypes.c_uint32), ("drop_philox", ctypes.c_int32),
         ("drop_bits", ctypes.c_void_p), ("drop_bits_filled", ctypes.c_int32), ("drop_mask_kind", ctypes.c_int32),
+        ("mask_bits", ctypes.c_void_p), ("mask_bits_filled", ctypes.c_int32), ("reserved0", ctypes.c_int32),
     ]
 
 
@@ -83,6 +84,8 @@ def load():
     lib.acct_fa_fwd_workspace_bytes.restype = ctypes.c_size_t
     lib.acct_fa_drop_bits_bytes.argtypes = [P]
     lib.acct_fa_drop_bits_bytes.restype = ctypes.c_size_t
+    lib.acct_fa_mask_bits_bytes.argtypes = [P]
+    lib.acct_fa_mask_bits_bytes.restype = ctypes.c_size_t
     lib.acct_fa_bwd_workspace_bytes.argtypes = [P]
     lib.acct_fa_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.acct_last_error.argtypes = []
@@ -215,6 +218,20 @@ def attach_drop_bits(p, device):
     buf = torch.empty(n, dtype=torch.uint8, device=device)
     p.drop_bits = buf.data_ptr()
     p.drop_bits_filled = 0
+    return buf
+
+
+def attach_mask_bits(p, device):
+    """Give `p` a buffer for what the pre-passes derive from its attn_mask (block classes, column bitmaps), so
+    that the first call of a step runs them once and the later calls read them: set `p.mask_bits_filled = 1`
+    after the first call.  Returns the buffer (the caller keeps it alive), or None when `p` has no mask tensor."""
+    lib = load()
+    n = lib.acct_fa_mask_bits_bytes(ctypes.byref(p))
+    if n == 0:
+        return None
+    buf = torch.empty(n, dtype=torch.uint8, device=device)
+    p.mask_bits = buf.data_ptr()
+    p.mask_bits_filled = 0
     return buf
 
 

@@ -132,6 +132,7 @@ int validate(const acct_fa_params* p, bool backward) {
   if (p->alibi && (p->alibi_stride_b < 0 || p->alibi_stride_h < 0 || p->alibi_stride_q < 0))
     return fail(ACCT_E_SHAPE, "alibi strides must be >= 0");
   if ((uintptr_t)p->drop_bits & 255) return fail(ACCT_E_WORKSPACE, "drop_bits must be 256-byte aligned");
+  if ((uintptr_t)p->mask_bits & 255) return fail(ACCT_E_WORKSPACE, "mask_bits must be 256-byte aligned");
   return ACCT_OK;
 }
 
@@ -170,11 +171,14 @@ acct::FaArgs make_args(const acct_fa_params* p) {
   }
   a.inv_scale = 1.0f / p->scale;
   {
-    // 2^p_shift grows with the key count (average probability 1 / Sk) and stops at 2^8, which leaves
-    // |dP - D| < 255 of headroom in fp16 for a row whose probability mass sits on one key
+    // 2^p_shift grows with the key count (average probability 1 / Sk): none up to 4096 keys, where P and
+    // dS = P (dP - D) sit in fp16's normal range by themselves and the overflow bound of dS is the reference's
+    // own (|dS| < 65504, its dS is fp16 too, flash_attention_bwd.py:161-181); one power of two per doubling of
+    // Sk after that, up to 2^8.  With a shift the bound is 65504 / 2^p_shift.  bf16 runs keep the shift: the
+    // P handed from the V-role to the K-role wave of the dK/dV kernel is fp16 in both cases.
     int lg = 0;
     while ((2 << lg) <= p->Sk) lg++;
-    const int sh = lg - 9 < 0 ? 0 : (lg - 9 > 8 ? 8 : lg - 9);
+    const int sh = lg - 12 < 0 ? 0 : (lg - 12 > 8 ? 8 : lg - 12);
     a.p_shift = (float)sh;
     a.p_unshift = 1.0f / (float)(1 << sh);
   }
@@ -187,15 +191,22 @@ acct::FaArgs make_args(const acct_fa_params* p) {
   return a;
 }
 
-size_t flag_bytes(const acct_fa_params* p) {
+// block classes of a dense mask (one byte per 128x128 block), then the scratch of the classification
+// pre-pass (16 bytes per block)
+size_t class_bytes(const acct_fa_params* p) {
   if (!mask_is_dense(p)) return 0;
   const size_t MB = p->mask_stride_b ? p->B : 1;
   return align_up(MB * (size_t)((p->Sq + 127) / 128) * (size_t)((p->Sk + 127) / 128), 256);
 }
-// classify the blocks of a dense mask; fills a.blkflags
+size_t flag_bytes(const acct_fa_params* p) {
+  if (!mask_is_dense(p)) return 0;
+  const size_t MB = p->mask_stride_b ? p->B : 1;
+  return class_bytes(p) + align_up(16 * MB * (size_t)((p->Sq + 127) / 128) * (size_t)((p->Sk + 127) / 128), 256);
+}
+// classify the blocks of a dense mask; fills a.blkflags (`flags`: flag_bytes(p) bytes)
 hipError_t prepare_mask(acct::FaArgs& a, const acct_fa_params* p, uint8_t* flags, hipStream_t st) {
   a.blkflags = flags;
-  return acct::launch_mask_blocks(a, flags, p->mask_stride_b ? p->B : 1, st);
+  return acct::launch_mask_blocks(a, flags, (uint32_t*)(flags + class_bytes(p)), p->mask_stride_b ? p->B : 1, st);
 }
 
 // per-key-column bitmaps of the mixed blocks of a dense mask (backward only): 16 bytes per (q block, key)
@@ -217,6 +228,32 @@ size_t dropcol_bytes(const acct_fa_params* p) {
   return align_up((size_t)p->B * p->N * (size_t)((p->Sq + 127) / 128) * (size_t)p->Sk * 16, 256);
 }
 
+// Pre-passes over the attention mask: block classes of a dense mask (all three kernels) and the mask packed by
+// key column (dK/dV kernel; also for the compact tile).  They run into `own` (a workspace region of
+// flag_bytes + colbit_bytes) or, when the caller lends a mask_bits buffer, once into that buffer: the call that
+// finds it unfilled runs BOTH pre-passes, whichever kernels it launches itself, so that the later calls of the
+// step only read.
+int mask_prepass(acct::FaArgs& a, const acct_fa_params* p, uint8_t* own, bool want_cols, hipStream_t st) {
+  if (!mask_is_dense(p) && !mask_is_tile(p)) return ACCT_OK;
+  uint8_t* base = p->mask_bits ? (uint8_t*)p->mask_bits : own;
+  uint8_t* flags = base;                                            // (no classes for the tile kind: flag_bytes = 0)
+  uint32_t* cbits = (uint32_t*)(base + flag_bytes(p));
+  const bool filled = p->mask_bits && p->mask_bits_filled;
+  const bool cols = p->mask_bits ? true : want_cols;
+  if (mask_is_dense(p)) a.blkflags = flags;
+  if (cols) a.colbits = cbits;
+  if (filled) return ACCT_OK;
+  if (mask_is_dense(p)) {
+    hipError_t e = prepare_mask(a, p, flags, st);
+    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
+  }
+  if (cols) {
+    hipError_t e = acct::launch_mask_colbits(a, flags, cbits, p->mask_stride_b ? p->B : 1, st);
+    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask bitmap kernel: %s", hipGetErrorString(e));
+  }
+  return ACCT_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -227,7 +264,12 @@ int acct_build_is_complete(void) { return acct::launch_variants_complete() ? 1 :
 
 size_t acct_fa_fwd_workspace_bytes(const acct_fa_params* p) {
   if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0 || p->Sk <= 0) return 0;
-  return flag_bytes(p) + (p->drop_bits ? 0 : droprow_bytes(p));
+  return (p->mask_bits ? 0 : flag_bytes(p)) + (p->drop_bits ? 0 : droprow_bytes(p));
+}
+
+size_t acct_fa_mask_bits_bytes(const acct_fa_params* p) {
+  if (!p || p->B <= 0 || p->N <= 0 || p->Sq <= 0 || p->Sk <= 0) return 0;
+  return flag_bytes(p) + colbit_bytes(p);
 }
 
 size_t acct_fa_drop_bits_bytes(const acct_fa_params* p) {
@@ -237,7 +279,7 @@ size_t acct_fa_drop_bits_bytes(const acct_fa_params* p) {
 
 // what the backward cannot do without: D and the exp2 offsets, the mask classes and bitmaps, the keep bits
 static size_t bwd_min_workspace_bytes(const acct_fa_params* p) {
-  return 2 * align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + flag_bytes(p) + colbit_bytes(p) +
+  return 2 * align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + (p->mask_bits ? 0 : flag_bytes(p) + colbit_bytes(p)) +
          (p->drop_bits ? 0 : droprow_bytes(p) + dropcol_bytes(p));
 }
 
@@ -266,13 +308,13 @@ int acct_fa_fwd(const acct_fa_params* p, void* O, float* LSE, void* workspace, s
   hipStream_t st = (hipStream_t)stream;
   acct::FaArgs a = make_args(p);
   a.o = O; a.lse = LSE;
-  if (mask_is_dense(p)) {
-    hipError_t e = prepare_mask(a, p, (uint8_t*)workspace, st);
-    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
+  {
+    rc = mask_prepass(a, p, (uint8_t*)workspace, /*want_cols=*/false, st);
+    if (rc) return rc;
   }
   if (dropout_on(p)) {
     // own bits by query row in the workspace, or both layouts in the caller's buffer for the backward call
-    uint32_t* rows = p->drop_bits ? (uint32_t*)p->drop_bits : (uint32_t*)((char*)workspace + flag_bytes(p));
+    uint32_t* rows = p->drop_bits ? (uint32_t*)p->drop_bits : (uint32_t*)((char*)workspace + (p->mask_bits ? 0 : flag_bytes(p)));
     uint32_t* cols = p->drop_bits ? (uint32_t*)((char*)p->drop_bits + droprow_bytes(p)) : nullptr;
     a.droprow = rows;
     a.droprow_w = (int)droprow_words(p);
@@ -315,21 +357,14 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
   const size_t stat_bytes = align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256);
   a.delta = (float*)workspace;
   a.nlse = (float*)((char*)workspace + stat_bytes);
-  if (mask_is_dense(p)) {
-    uint8_t* flags = (uint8_t*)workspace + 2 * stat_bytes;
-    // (the dkdv-only call re-derives the flags as well: the mask may have been edited since)
-    hipError_t e = prepare_mask(a, p, flags, st);
-    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
-  }
-  if (want_dkdv && (mask_is_dense(p) || mask_is_tile(p))) {
-    uint8_t* flags = (uint8_t*)workspace + 2 * stat_bytes;          // (no flags for the tile kind: flag_bytes = 0)
-    uint32_t* cbits = (uint32_t*)(flags + flag_bytes(p));
-    a.colbits = cbits;
-    hipError_t e = acct::launch_mask_colbits(a, flags, cbits, p->mask_stride_b ? p->B : 1, st);
-    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask bitmap kernel: %s", hipGetErrorString(e));
+  {
+    // (without a caller-held mask_bits buffer the dkdv-only call re-derives the classes as well: the mask may
+    // have been edited since)
+    rc = mask_prepass(a, p, (uint8_t*)workspace + 2 * stat_bytes, want_dkdv, st);
+    if (rc) return rc;
   }
   if (dropout_on(p)) {
-    char* base = p->drop_bits ? (char*)p->drop_bits : (char*)workspace + 2 * stat_bytes + flag_bytes(p) + colbit_bytes(p);
+    char* base = p->drop_bits ? (char*)p->drop_bits : (char*)workspace + 2 * stat_bytes + (p->mask_bits ? 0 : flag_bytes(p) + colbit_bytes(p));
     uint32_t* rows = (uint32_t*)base;
     uint32_t* cols = (uint32_t*)(base + droprow_bytes(p));
     a.droprow = rows;
@@ -349,7 +384,7 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
   }
   a.q_split = 1;
   if (want_dkdv) {
-    const acct::DkdvSplit sp = acct::dkdv_split(p->B, p->N, p->Sq, p->Sk, p->D);
+    const acct::DkdvSplit sp = acct::dkdv_split(p->B, p->N, p->Sq, p->Sk, p->D, n_cu);
     const size_t part_at = align_up(need, 256);
     if (sp.q_split > 1 && workspace_bytes >= part_at + sp.part_bytes) {
       a.q_split = sp.q_split;

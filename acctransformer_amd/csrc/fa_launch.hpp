@@ -34,12 +34,14 @@ inline int head_dim_class(int D) {
 // few heads and a short key sequence (cross attention on 77 keys) that is a handful of workgroups for 256 CUs:
 // the query range is then cut into q_split slices that run side by side, and a second kernel adds their sums.
 // Returns q_split (1 = no split) and the bytes of workspace the slices' sums take.
+// `n_cu`: compute units of the device that runs the launch; the workspace-size query passes the 256 of a whole
+// MI355X, which is also the upper bound of what a partition of it asks for.
 struct DkdvSplit { int q_split; size_t part_bytes; };
-inline DkdvSplit dkdv_split(int B, int N, int Sq, int Sk, int D) {
+inline DkdvSplit dkdv_split(int B, int N, int Sq, int Sk, int D, int n_cu = 256) {
   const int dc = head_dim_class(D), ngk = dc > 128 ? 1 : 2, db = (dc + 31) / 32;
   const long long n_wg = (long long)B * N * ((Sk + 128 * ngk - 1) / (128 * ngk));
   const long long tiles64 = (Sq + 63) / 64;
-  long long s = 256 / n_wg;                          // (the CU count of the one part this library is built for)
+  long long s = (n_cu > 256 ? 256 : n_cu) / n_wg;
   if (tiles64 / 8 < s) s = tiles64 / 8;              // a slice keeps at least 512 query rows
   if (s > 16) s = 16;
   if (s < 2) return {1, 0};
@@ -57,8 +59,9 @@ hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t
 // false when the kernel translation units were compiled with a reduced variant set (ACCT_DEV_BUILD)
 bool launch_variants_complete();
 
-// classify the 128x128 blocks of a dense uint8 mask into clean / apply / skip
-hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, int MB, hipStream_t st);
+// classify the 128x128 blocks of a dense mask into clean / apply / skip / causal diagonal; `scan` is scratch of
+// 16 bytes per block (per-row "has an unmasked element" bits between the two launches of the fast path)
+hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, uint32_t* scan, int MB, hipStream_t st);
 // pack the dropout mask into keep bits by query row [B*N, Sq, droprow_w] and / or by key column [B*N, Tr, Sk, 4]
 hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st);
 // the same two bitmaps generated from (a.philox_k0, a.philox_k1, a.philox_offset, a.philox_thr) instead of read from a mask

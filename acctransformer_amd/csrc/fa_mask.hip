@@ -18,93 +18,106 @@ namespace acct {
 
 constexpr uint8_t kBlkAllMasked = 255;  // provisional: resolved to skip or apply below
 
-// Fast path (Sk and the mask pointers 16-byte aligned, at most 64 column blocks per pass): one
-// workgroup of 1024 threads per (mask batch, q block); thread t owns the 16-byte piece t%8 of row
-// t/8 of every 128x128 block, so a block is one 16-byte load per thread and many blocks are in
-// flight at once.  Per-block "any masked" / "any unmasked" bits are gathered in two 64-bit masks
-// and reduced once at the end.
+// Fast path (Sk and the mask pointers 16-byte aligned), in two launches so that the work spreads over the
+// chip whatever the shape (a [1, 2048, 2048] mask has 16 row blocks but 256 blocks):
+//
+// fa_mask_scan_kernel: one workgroup of 256 threads per (mask batch, q block, key block) inside the band.
+// Thread t owns 64 consecutive elements of row t % 128 (half t / 128 of the block's 128 columns), four or
+// eight 16-byte loads.  It leaves the block's provisional class (clean / apply / all masked / the causal
+// diagonal pattern) and, per row, whether the row has an unmasked element in this block (128 bits).
+//
+// fa_mask_resolve_kernel: one wave per (mask batch, q block) ORs those row bits over the band and turns
+// "all masked" into skip when every row of the q block has an unmasked key somewhere, else into apply.
 template <int ES>
-__global__ void __launch_bounds__(1024) fa_mask_blocks_vec_kernel(const FaArgs a, uint8_t* flags) {
-  __shared__ unsigned long long s_m, s_u;
-  const int qb = blockIdx.x % a.Tr, mb = blockIdx.x / a.Tr;
-  const int tid = threadIdx.x, row = qb * 128 + (tid >> 3), c0 = (tid & 7) * 16;
-  const uint8_t* mrow = a.mask + ((int64_t)mb * a.mask_sb + (int64_t)min(row, a.Sq - 1) * a.Sk) * ES;
-  uint8_t* frow = flags + ((int64_t)mb * a.Tr + qb) * a.Tc;
+__global__ void __launch_bounds__(256) fa_mask_scan_kernel(const FaArgs a, uint8_t* flags, uint32_t* rowseen) {
+  __shared__ unsigned long long s_seen[2];
+  const int kvb = blockIdx.x % a.Tc, qb = (blockIdx.x / a.Tc) % a.Tr, mb = blockIdx.x / (a.Tc * a.Tr);
+  const int tid = threadIdx.x;
   int lo = max(0, qb - a.prev_blk), hi = min(a.Tc - 1, qb + a.next_blk);
   if (a.row_prefix) hi = min(hi, ((qb * 128 / a.row_prefix + 1) * a.row_prefix - 1) / 128);
-  for (int kvb = tid; kvb < a.Tc; kvb += 1024)
-    if (kvb < lo || kvb > hi) frow[kvb] = kBlkClean;
-  bool row_unmasked = false;
-  bool tri_bad = false;                                 // the diagonal block differs from "key after query"
-  for (int base = lo; base <= hi; base += 64) {        // 64 column blocks per pass
-    if (tid == 0) { s_m = 0; s_u = 0; }
-    __syncthreads();
-    unsigned long long bm = 0, bu = 0;
-    const int n = min(64, hi - base + 1);
-    if (row < a.Sq) {
-#pragma unroll 8
-      for (int i = 0; i < n; i++) {
-        const int kv = (base + i) * 128 + c0;
-        if (kv < a.Sk) {                                // Sk % 16 == 0: a piece is entirely inside or outside
-          bool has_zero = false, has_nonzero = false;
-          const bool on_diag = base + i == qb;          // the per-element pattern matters on the diagonal block only
-          uint32_t nz = 0;                              // bit e: element e of this thread's 16 is nonzero
+  const int64_t blk = ((int64_t)mb * a.Tr + qb) * a.Tc + kvb;
+  if (kvb < lo || kvb > hi) {                           // outside the band: never visited
+    if (tid == 0) flags[blk] = kBlkClean;
+    return;
+  }
+  if (tid < 2) s_seen[tid] = 0;
+  __syncthreads();
+  const int rib = tid & 127, half = tid >> 7, row = qb * 128 + rib, c0 = half * 64;
+  const uint8_t* mrow = a.mask + ((int64_t)mb * a.mask_sb + (int64_t)min(row, a.Sq - 1) * a.Sk) * ES;
+  const bool on_diag = kvb == qb;                       // the per-element pattern matters on the diagonal block only
+  bool has_zero = false, has_nonzero = false, tri_bad = false;
+  if (row < a.Sq) {
 #pragma unroll
-          for (int h = 0; h < ES; h++) {
-            const u32x4 v = *reinterpret_cast<const u32x4*>(mrow + (int64_t)kv * ES + 16 * h);
+    for (int i = 0; i < 4; i++) {
+      const int col = c0 + 16 * i, kv = kvb * 128 + col;
+      if (kv < a.Sk) {                                  // Sk % 16 == 0: a piece is entirely inside or outside
+        uint32_t nz = 0;                                // bit e: element e of these 16 is nonzero
 #pragma unroll
-            for (int w = 0; w < 4; w++) {
-              if (ES == 1) {
-                // a byte is zero iff (x - 0x01010101) & ~x & 0x80808080 has its top bit set
-                has_nonzero |= v[w] != 0;
-                has_zero |= ((v[w] - 0x01010101u) & ~v[w] & 0x80808080u) != 0;
-                if (on_diag) {
+        for (int h = 0; h < ES; h++) {
+          const u32x4 v = *reinterpret_cast<const u32x4*>(mrow + (int64_t)kv * ES + 16 * h);
 #pragma unroll
-                  for (int e = 0; e < 4; e++) nz |= (((v[w] >> (8 * e)) & 0xffu) != 0 ? 1u : 0u) << (4 * w + e);
-                }
-              } else {
-                // 2-byte floating-point elements: the sign of a zero does not count
-                const uint32_t lo16 = v[w] & 0x7fffu, hi16 = (v[w] >> 16) & 0x7fffu;
-                has_nonzero |= (lo16 | hi16) != 0;
-                has_zero |= lo16 == 0 || hi16 == 0;
-                if (on_diag) nz |= ((lo16 != 0 ? 1u : 0u) | (hi16 != 0 ? 2u : 0u)) << (8 * h + 2 * w);
+          for (int w = 0; w < 4; w++) {
+            if (ES == 1) {
+              // a byte is zero iff (x - 0x01010101) & ~x & 0x80808080 has its top bit set
+              has_nonzero |= v[w] != 0;
+              has_zero |= ((v[w] - 0x01010101u) & ~v[w] & 0x80808080u) != 0;
+              if (on_diag) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) nz |= (((v[w] >> (8 * e)) & 0xffu) != 0 ? 1u : 0u) << (4 * w + e);
               }
+            } else {
+              // 2-byte floating-point elements: the sign of a zero does not count
+              const uint32_t lo16 = v[w] & 0x7fffu, hi16 = (v[w] >> 16) & 0x7fffu;
+              has_nonzero |= (lo16 | hi16) != 0;
+              has_zero |= lo16 == 0 || hi16 == 0;
+              if (on_diag) nz |= ((lo16 != 0 ? 1u : 0u) | (hi16 != 0 ? 2u : 0u)) << (8 * h + 2 * w);
             }
           }
-          if (has_nonzero) bm |= 1ull << i;
-          if (has_zero) bu |= 1ull << i;
-          if (on_diag) {
+        }
+        if (on_diag) {
 #pragma unroll
-            for (int e = 0; e < 16; e++) tri_bad |= (((nz >> e) & 1u) != 0) != (c0 + e > (tid >> 3));
-          }
+          for (int e = 0; e < 16; e++) tri_bad |= (((nz >> e) & 1u) != 0) != (col + e > rib);
         }
       }
     }
-    row_unmasked |= bu != 0;
-    // wave-level OR, then one LDS atomic per wave
+  }
+  // rows 64 (tid / 64 % 2) .. +63 of the block: one ballot per wave, the two column halves OR-ed in LDS
+  const unsigned long long seen = __ballot(has_zero);
+  if ((tid & 63) == 0) atomicOr(&s_seen[(tid >> 6) & 1], seen);
+  const int any_m = __syncthreads_or(has_nonzero), any_u = __syncthreads_or(has_zero), bad = __syncthreads_or(tri_bad);
+  if (tid < 4) rowseen[blk * 4 + tid] = (uint32_t)(s_seen[tid >> 1] >> (32 * (tid & 1)));
+  if (tid == 0) flags[blk] = !any_m ? kBlkClean : (!any_u ? kBlkAllMasked : ((on_diag && !bad) ? kBlkTriu : kBlkApply));
+}
+
+__global__ void __launch_bounds__(64) fa_mask_resolve_kernel(const FaArgs a, uint8_t* flags, const uint32_t* rowseen) {
+  const int qb = blockIdx.x % a.Tr, mb = blockIdx.x / a.Tr, lane = threadIdx.x;
+  int lo = max(0, qb - a.prev_blk), hi = min(a.Tc - 1, qb + a.next_blk);
+  if (a.row_prefix) hi = min(hi, ((qb * 128 / a.row_prefix + 1) * a.row_prefix - 1) / 128);
+  uint8_t* frow = flags + ((int64_t)mb * a.Tr + qb) * a.Tc;
+  const u32x4* seen = reinterpret_cast<const u32x4*>(rowseen) + ((int64_t)mb * a.Tr + qb) * a.Tc;
+  u32x4 acc = {0u, 0u, 0u, 0u};
+  bool any_allmasked = false;
+  for (int kvb = lo + lane; kvb <= hi; kvb += 64) {
+    const u32x4 v = seen[kvb];
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      bm |= __shfl_xor(bm, off);
-      bu |= __shfl_xor(bu, off);
-    }
-    if ((tid & 63) == 0) { atomicOr(&s_m, bm); atomicOr(&s_u, bu); }
-    __syncthreads();
-    for (int i = tid; i < n; i += 1024) {
-      const bool blk_m = (s_m >> i) & 1, blk_u = (s_u >> i) & 1;
-      frow[base + i] = !blk_m ? kBlkClean : (!blk_u ? kBlkAllMasked : kBlkApply);
-    }
-    __syncthreads();
+    for (int w = 0; w < 4; w++) acc[w] |= v[w];
+    any_allmasked |= frow[kvb] == kBlkAllMasked;
   }
-  // a row is covered if any of its 8 threads saw an unmasked byte
-  row_unmasked |= (bool)__shfl_xor((int)row_unmasked, 1);
-  row_unmasked |= (bool)__shfl_xor((int)row_unmasked, 2);
-  row_unmasked |= (bool)__shfl_xor((int)row_unmasked, 4);
-  const int rows_ok = __syncthreads_and(row >= a.Sq || row_unmasked);
-  const int not_tri = __syncthreads_or(tri_bad);
-  for (int kvb = lo + tid; kvb <= hi; kvb += 1024) {
+  if (!__any(any_allmasked)) return;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1)
+#pragma unroll
+    for (int w = 0; w < 4; w++) acc[w] |= (uint32_t)__shfl_xor((int)acc[w], off);
+  const int nrow = min(128, a.Sq - qb * 128);           // rows past Sq do not count
+  bool rows_ok = true;
+#pragma unroll
+  for (int w = 0; w < 4; w++) {
+    const int n = min(32, max(0, nrow - 32 * w));
+    const uint32_t need = n >= 32 ? 0xffffffffu : ((1u << n) - 1u);
+    rows_ok = rows_ok && (acc[w] & need) == need;
+  }
+  for (int kvb = lo + lane; kvb <= hi; kvb += 64)
     if (frow[kvb] == kBlkAllMasked) frow[kvb] = rows_ok ? kBlkSkip : kBlkApply;
-    else if (kvb == qb && frow[kvb] == kBlkApply && !not_tri) frow[kvb] = kBlkTriu;
-  }
 }
 
 // Generic path (any alignment): one workgroup per (mask batch, q block); thread t scans 64 columns of row t/2
@@ -324,17 +337,21 @@ hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbit
   return hipGetLastError();
 }
 
-hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, int MB, hipStream_t st) {
+hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, uint32_t* scan, int MB, hipStream_t st) {
   // fast path: every 16-element piece of a row is 16-byte aligned and entirely inside or outside the row
   const bool vec = (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 15) == 0;
-  const dim3 grid((unsigned)(MB * a.Tr));
-  if (a.mask_es == 2) {
-    if (vec) hipLaunchKernelGGL(fa_mask_blocks_vec_kernel<2>, grid, dim3(1024), 0, st, a, flags);
-    else hipLaunchKernelGGL(fa_mask_blocks_kernel<2>, grid, dim3(256), 0, st, a, flags);
-  } else {
-    if (vec) hipLaunchKernelGGL(fa_mask_blocks_vec_kernel<1>, grid, dim3(1024), 0, st, a, flags);
-    else hipLaunchKernelGGL(fa_mask_blocks_kernel<1>, grid, dim3(256), 0, st, a, flags);
+  if (vec) {
+    const dim3 grid((unsigned)((long long)MB * a.Tr * a.Tc));
+    if (a.mask_es == 2) hipLaunchKernelGGL(fa_mask_scan_kernel<2>, grid, dim3(256), 0, st, a, flags, scan);
+    else hipLaunchKernelGGL(fa_mask_scan_kernel<1>, grid, dim3(256), 0, st, a, flags, scan);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(fa_mask_resolve_kernel, dim3((unsigned)(MB * a.Tr)), dim3(64), 0, st, a, flags, (const uint32_t*)scan);
+    return hipGetLastError();
   }
+  const dim3 grid((unsigned)(MB * a.Tr));
+  if (a.mask_es == 2) hipLaunchKernelGGL(fa_mask_blocks_kernel<2>, grid, dim3(256), 0, st, a, flags);
+  else hipLaunchKernelGGL(fa_mask_blocks_kernel<1>, grid, dim3(256), 0, st, a, flags);
   return hipGetLastError();
 }
 

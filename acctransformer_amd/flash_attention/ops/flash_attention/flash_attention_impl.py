@@ -59,7 +59,11 @@ def _is_compact_shape(shape):
     return False
 
 
-DETECT_CAUSAL_MASKS = True     # look once per mask tensor whether it is the plain causal mask (one device compare, one sync)
+# Off (the default): an attn_mask tensor goes to the library as it is, and the library's own pre-pass finds the
+# blocks that are clean, wholly masked or the plain causal diagonal -- on the device, with no host round trip.
+# On: the operator compares the mask with the lower-triangular pattern once per tensor (one device compare and
+# one host sync) and, on a match, passes ACCT_MASK_CAUSAL, which needs no pre-pass at all.
+DETECT_CAUSAL_MASKS = False
 
 
 def _classify_mask(attn_mask, Sq, Sk, io_dtype):
@@ -69,7 +73,8 @@ def _classify_mask(attn_mask, Sq, Sk, io_dtype):
     version, so a mask reused across steps is inspected once."""
     key = id(attn_mask)
     hit = _mask_cache.get(key)
-    if hit is not None and hit[0]() is attn_mask and hit[1] == attn_mask._version and hit[2] == (Sq, Sk, io_dtype):
+    if (hit is not None and hit[0]() is attn_mask and hit[1] == attn_mask._version
+            and hit[2] == (Sq, Sk, io_dtype, DETECT_CAUSAL_MASKS)):
         return hit[3], hit[4]
     if attn_mask.dtype == torch.bool:
         m = attn_mask.contiguous().view(torch.uint8)
@@ -81,11 +86,11 @@ def _classify_mask(attn_mask, Sq, Sk, io_dtype):
     compact = _is_compact_shape(tuple(attn_mask.shape)) and not (Sq == TILING_BLOCK_SIZE and Sk == TILING_BLOCK_SIZE
                                                                   and attn_mask.dim() == 3)
     if compact:
-        tri = torch.triu(torch.ones(128, 128, dtype=torch.bool, device=m.device), diagonal=1)
-        if torch.equal(m.reshape(128, 128).ne(0), tri):
-            kind, out = _capi.MASK_CAUSAL, None      # evaluated by index compare, no loads
-        else:
-            kind, out = (_capi.MASK_TILE_F16 if wide else _capi.MASK_TILE_U8), m.reshape(128, 128)
+        kind, out = (_capi.MASK_TILE_F16 if wide else _capi.MASK_TILE_U8), m.reshape(128, 128)
+        if DETECT_CAUSAL_MASKS:
+            tri = torch.triu(torch.ones(128, 128, dtype=torch.bool, device=m.device), diagonal=1)
+            if torch.equal(m.reshape(128, 128).ne(0), tri):
+                kind, out = _capi.MASK_CAUSAL, None      # evaluated by index compare, no loads
         compact_kind = True
     else:
         compact_kind = False
@@ -102,8 +107,51 @@ def _classify_mask(attn_mask, Sq, Sk, io_dtype):
     if len(_mask_cache) > 64:
         for k_ in [k_ for k_, v_ in _mask_cache.items() if v_[0]() is None]:
             del _mask_cache[k_]
-    _mask_cache[key] = (weakref.ref(attn_mask), attn_mask._version, (Sq, Sk, io_dtype), kind, out, compact_kind)
+    _mask_cache[key] = (weakref.ref(attn_mask), attn_mask._version, (Sq, Sk, io_dtype, DETECT_CAUSAL_MASKS), kind, out, compact_kind)
     return kind, out
+
+
+# ---- what the library's pre-passes derive from a mask tensor, kept per tensor ----
+# Block classes and column bitmaps depend on the mask's contents and on the band only, so a mask that is
+# reused from step to step (the usual case) is classified once: the buffer is handed to every later call
+# with mask_bits_filled = 1.  Entries are dropped with their tensor, on an in-place edit of it (torch's
+# version counter), and when a call arrives on another stream (the fill is ordered on the stream that ran it).
+_mask_bits_cache = {}
+
+
+def _attach_mask_bits(p, mask_tensor, device):
+    """Points `p` at the pre-pass results of `mask_tensor` (the tensor handed to the library): a filled buffer
+    from an earlier call, or a fresh one that `_mask_bits_done(p)` marks as filled once a call has run."""
+    if p.mask_kind not in (_capi.MASK_DENSE_U8, _capi.MASK_DENSE_F16, _capi.MASK_TILE_U8, _capi.MASK_TILE_F16):
+        return
+    stream = torch.cuda.current_stream(device).cuda_stream
+    sig = (p.mask_kind, p.B, p.Sq, p.Sk, p.prev_block_num, p.next_block_num, p.row_block_prefix, stream,
+           mask_tensor.data_ptr())
+    key = id(mask_tensor)
+    hit = _mask_bits_cache.get(key)
+    if hit is not None and hit[0]() is mask_tensor and hit[1] == mask_tensor._version and hit[2] == sig:
+        entry = hit
+    else:
+        buf = _capi.attach_mask_bits(p, device)
+        if buf is None:
+            return
+        if len(_mask_bits_cache) > 64:
+            for k_ in [k_ for k_, v_ in _mask_bits_cache.items() if v_[0]() is None]:
+                del _mask_bits_cache[k_]
+        entry = (weakref.ref(mask_tensor), mask_tensor._version, sig, buf, [False])
+        _mask_bits_cache[key] = entry
+    p.mask_bits = entry[3].data_ptr()
+    p.mask_bits_filled = 1 if entry[4][0] else 0
+    p._keepalive.append(entry[3])
+    p._mask_bits_entry = entry
+
+
+def _mask_bits_done(p):
+    """A call with `p` has been enqueued: its mask pre-pass results are in the buffer for every later call."""
+    entry = getattr(p, "_mask_bits_entry", None)
+    if entry is not None:
+        entry[4][0] = True
+        p.mask_bits_filled = 1
 
 
 def _is_seed_pair(x):
@@ -145,10 +193,14 @@ def _build_params(q, k, v, attn_mask, dropout_mask, alibi_mask, prev_block_num, 
     d8, keep, seed = _prepare_dropout(dropout_mask, keep_prob, q.dtype)
     if alibi_mask is not None and alibi_mask.dtype != q.dtype:
         alibi_mask = alibi_mask.to(q.dtype)
-    return _capi.make_params(q, k, v, scale=scale, keep_prob=keep, prev_block_num=prev_block_num,
-                             next_block_num=next_block_num, mask_kind=kind, attn_mask=m8, drop_mask=d8,
-                             alibi=alibi_mask, row_block_prefix=row_block_prefix,
-                             drop_seed=None if seed is None else seed[0], drop_offset=0 if seed is None else seed[1])
+    p = _capi.make_params(q, k, v, scale=scale, keep_prob=keep, prev_block_num=prev_block_num,
+                          next_block_num=next_block_num, mask_kind=kind, attn_mask=m8, drop_mask=d8,
+                          alibi=alibi_mask, row_block_prefix=row_block_prefix,
+                          drop_seed=None if seed is None else seed[0], drop_offset=0 if seed is None else seed[1])
+    if m8 is not None and q.is_cuda:
+        # block classes / column bitmaps of the mask: derived once per mask tensor, by the first call that sees it
+        _attach_mask_bits(p, m8, q.device)
+    return p
 
 
 def _rows_contiguous(t):
@@ -166,6 +218,7 @@ class _FlashAttentionFn(torch.autograd.Function):
         needs_grad = any(ctx.needs_input_grad[:3])
         ctx.drop_bits = _capi.attach_drop_bits(p, q.device) if needs_grad else None
         o, lse = _capi.fa_fwd(p, q)
+        _mask_bits_done(p)
         if ctx.drop_bits is not None:
             p.drop_bits_filled = 1
         ctx.save_for_backward(q, k, v, o, lse)
@@ -194,6 +247,7 @@ def get_flash_attention_grad(prev_block_num=65536, next_block_num=65536, tiling_
         p = _build_params(q, k, v, attn_mask, dropout_mask, alibi_mask, prev_block_num, next_block_num, scale, keep_prob,
                           row_block_prefix)
         dq, dk, dv = _capi.fa_bwd(p, q, k, v, output, dout, rowsum)
+        _mask_bits_done(p)
         zeros = tuple(torch.zeros_like(t) if torch.is_tensor(t) else None for t in (attn_mask, dropout_mask, alibi_mask))
         return (dq, dk, dv) + zeros
 

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define ACCT_FA_VERSION 107
+#define ACCT_FA_VERSION 108
 
 /* error codes (0 = success) */
 #define ACCT_OK          0
@@ -125,6 +125,20 @@ typedef struct acct_fa_params {
   void*    drop_bits;
   int32_t  drop_bits_filled;
   int32_t  drop_mask_kind;       /* ACCT_DROP_* (field added in version 104; 0 = the uint8 form) */
+  /* What the pre-passes derive from attn_mask, shared between the calls of one training step (fields added in
+     version 108; no counterpart in the reference, whose kernels read the mask tile by tile,
+     T/attention.py:357-371).  A dense mask is classified block by block (clean / apply / skip / causal
+     diagonal) and, for the dK/dV kernel, packed by key column; the compact tile is packed by key column.
+     With mask_bits == NULL every call runs the pre-passes into its own workspace.  With mask_bits pointing
+     at acct_fa_mask_bits_bytes(p) bytes of device memory (256-byte aligned) that the caller keeps across the
+     calls, a call with mask_bits_filled == 0 runs them into that buffer and a call with
+     mask_bits_filled != 0 only reads it.  The caller sets mask_bits_filled after the first call returns, and
+     clears it when the contents of attn_mask change; the bits depend on attn_mask, mask_kind, B, Sq, Sk,
+     prev_block_num, next_block_num and row_block_prefix only, so a mask that stays the same from step to
+     step needs them once. */
+  void*    mask_bits;
+  int32_t  mask_bits_filled;
+  int32_t  reserved0;            /* must be 0 */
 } acct_fa_params;
 
 /* Forward: replaces the `flash_attention` TBE custom op, T/flash_attention_fwd.py:498-530
@@ -138,6 +152,9 @@ size_t acct_fa_fwd_workspace_bytes(const acct_fa_params* p);
 /* Size of the optional drop_bits buffer (0 without dropout): keep bits by query row for the forward and dQ
  * kernels, then by key column for the dK/dV kernel, a quarter of a byte per score in total. */
 size_t acct_fa_drop_bits_bytes(const acct_fa_params* p);
+
+/* Size of the optional mask_bits buffer (0 without an attn_mask tensor). */
+size_t acct_fa_mask_bits_bytes(const acct_fa_params* p);
 
 /* Backward: replaces the `flash_attention_grad` TBE custom op,
  * T/flash_attention_bwd.py:436-477 (the bprop of T/flash_attention_impl.py:117-124

@@ -521,6 +521,87 @@ def test_keep_bits_shared_between_forward_and_backward(source):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("form", ["dense_u8", "dense_f16", "tile_u8", "dense_u8_unaligned"])
+def test_mask_bits_shared_between_the_calls_of_a_step(form):
+    # The first call that finds the caller-held mask_bits buffer unfilled runs the mask pre-passes (block classes,
+    # column bitmaps) into it; the later calls of the step, and later steps on the same mask, only read it.  Every
+    # result equals, bit for bit, that of calls that each run the pre-passes into their own workspace.
+    B, N, D = 2, 3, 128
+    S = 333 if form == "dense_u8_unaligned" else 384
+    q, k, v, dO = (_gen((B, N, S, D), s).to(DEV) for s in (201, 202, 203, 204))
+    if form == "tile_u8":
+        mask = torch.triu(torch.ones(128, 128, dtype=torch.uint8), 1)
+        mask[5, 3] = 1
+        kw = dict(mask_kind=_capi.MASK_TILE_U8, attn_mask=mask.to(DEV), next_block_num=0)
+    else:
+        m = np.broadcast_to(np.triu(np.ones((S, S), np.uint8), 1), (B, S, S)).copy()
+        m[0, :, 300:] = 1                                  # padding: wholly masked and mixed blocks besides the diagonal
+        m[1, 200, 131] = 1                                 # a diagonal block that is not the causal pattern
+        mt = torch.from_numpy(m)
+        kw = dict(mask_kind=_capi.MASK_DENSE_F16 if form == "dense_f16" else _capi.MASK_DENSE_U8,
+                  attn_mask=(mt.half() if form == "dense_f16" else mt).to(DEV))
+    kw.update(scale=D ** -0.5)
+    lib = _capi.load()
+    p0 = _capi.make_params(q, k, v, **kw)
+    o0, lse0 = _capi.fa_fwd(p0, q)
+    g0 = _capi.fa_bwd(p0, q, k, v, o0, dO, lse0)
+
+    p1 = _capi.make_params(q, k, v, **kw)
+    bits = _capi.attach_mask_bits(p1, q.device)
+    assert bits is not None and bits.numel() == lib.acct_fa_mask_bits_bytes(ctypes.byref(p1))
+    assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p1)) == 0
+    bits.fill_(0xA5)                                       # whatever was there before is overwritten
+    o1, lse1 = _capi.fa_fwd(p1, q)
+    p1.mask_bits_filled = 1
+    torch.cuda.synchronize()
+    snapshot = bits.clone()
+    g1 = _capi.fa_bwd(p1, q, k, v, o1, dO, lse1)
+    o1b, lse1b = _capi.fa_fwd(p1, q)                       # a later step on the same mask
+    torch.cuda.synchronize()
+    assert torch.equal(bits, snapshot)                     # a filled buffer is only read
+    assert torch.equal(o0, o1) and torch.equal(lse0, lse1) and torch.equal(o0, o1b) and torch.equal(lse0, lse1b)
+    for a, b in zip(g0, g1):
+        assert torch.equal(a, b)
+
+    p2 = _capi.make_params(q, k, v, **kw)                  # backward first: it fills the buffer completely
+    bits2 = _capi.attach_mask_bits(p2, q.device)
+    g2 = _capi.fa_bwd(p2, q, k, v, o0, dO, lse0)
+    p2.mask_bits_filled = 1
+    o2, lse2 = _capi.fa_fwd(p2, q)
+    assert bits2 is not None and torch.equal(o0, o2)
+    for a, b in zip(g0, g2):
+        assert torch.equal(a, b)
+
+
+def test_operator_derives_the_mask_bits_once_per_mask_tensor():
+    # the Python operator keeps the pre-pass results with the mask tensor: the second step reads them, an in-place
+    # edit of the mask (torch's version counter) makes the next call derive them again -- no host sync either way
+    from acctransformer_amd.flash_attention.ops.flash_attention import flash_attention_impl as impl
+    B, N, S, D = 1, 2, 384, 64
+    q, k, v, dO = (_gen((B, N, S, D), s) for s in (205, 206, 207, 208))
+    m = np.triu(np.ones((1, S, S), np.uint8), 1)
+    md = torch.from_numpy(m).to(DEV)
+    fa = get_flash_attention(scale=D ** -0.5)
+    outs = []
+    for step in range(3):
+        if step == 2:
+            md[0, :, 300:] = 1                             # the mask changes in place
+            m[0, :, 300:] = 1
+        qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+        o, lse = fa(qd, kd, vd, md)
+        node = o.grad_fn
+        assert node.params.mask_kind == _capi.MASK_DENSE_U8 and node.params.mask_bits
+        assert node.params.mask_bits_filled == 1
+        entry = node.params._mask_bits_entry
+        outs.append((o.detach().clone(), entry))
+        o.backward(dO.to(DEV))
+        torch.cuda.synchronize()
+        _check_all(q, k, v, dO, dict(scale=D ** -0.5, attn_mask=m), (o, lse, (qd.grad, kd.grad, vd.grad)))
+    assert outs[0][1] is outs[1][1] and outs[1][1] is not outs[2][1]      # same buffer until the edit
+    assert torch.equal(outs[0][0], outs[1][0]) and not torch.equal(outs[1][0], outs[2][0])
+    assert not impl.DETECT_CAUSAL_MASKS
+
+
 def test_autograd_function_keeps_the_keep_bits_for_backward():
     B, N, S, D = 1, 2, 256, 64
     q, k, v, dO = (_gen((B, N, S, D), s).to(DEV) for s in (106, 107, 108, 109))

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     decl = re.findall(r"^\s*(?:int|size_t|const char\*)\s+(acct_\w+)\s*\(", _header(), flags=re.M)
     assert set(decl) >= {"acct_fa_fwd", "acct_fa_bwd", "acct_fa_bwd_dq", "acct_fa_bwd_dkdv",
                          "acct_fa_fwd_workspace_bytes", "acct_fa_bwd_workspace_bytes", "acct_last_error", "acct_version",
-                         "acct_fa_infer_shape", "acct_build_is_complete", "acct_fa_drop_bits_bytes"}
+                         "acct_fa_infer_shape", "acct_build_is_complete", "acct_fa_drop_bits_bytes", "acct_fa_mask_bits_bytes"}
     for name in decl:
         assert hasattr(lib, name), name
     m = re.search(r"#define ACCT_FA_VERSION (\d+)", _header())
@@ -49,7 +49,7 @@ def test_struct_mirror_matches_header_field_order():
         for part in decl.split(","):
             names.append(re.sub(r"\[\d+\]", "", part.strip().split()[-1]).lstrip("*"))
     assert names == [f[0] for f in _capi.AcctFaParams._fields_]
-    assert ctypes.sizeof(_capi.AcctFaParams) == 256
+    assert ctypes.sizeof(_capi.AcctFaParams) == 272
 
 
 def _params(**over):
@@ -87,13 +87,23 @@ def test_null_outputs_and_workspace_sizes():
     m = torch.zeros(1, 128, 128, dtype=torch.uint8)
     q = torch.zeros(2, 2, 128, 128, dtype=torch.float16)
     p2 = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m)
-    assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p2)) == 256
+    # block classes (padded to 256) and the classification pre-pass's scratch (16 bytes per block, padded)
+    assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p2)) == 256 + 256
     raw = (ctypes.c_char * 128)()
     addr = (ctypes.addressof(raw) + 63) // 64 * 64
     # backward without its workspace is refused before any launch
     assert lib.acct_fa_bwd(ctypes.byref(p2), *([addr] * 6), None, 0, None) == -7
-    # D and -LSE*log2e rows, block classes (padded to 256), key-column bitmaps: 16 bytes per (q block, key)
-    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p2)) == 2 * (2 * 2 * 128 * 4) + 256 + 1 * 1 * 128 * 16
+    # D and -LSE*log2e rows, block classes + scratch (padded to 256 each), key-column bitmaps: 16 bytes per (q block, key)
+    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p2)) == 2 * (2 * 2 * 128 * 4) + 512 + 1 * 1 * 128 * 16
+    # a caller-held mask_bits buffer takes the classes, the scratch and the bitmaps out of both workspaces
+    assert lib.acct_fa_mask_bits_bytes(ctypes.byref(p2)) == 512 + 128 * 16
+    assert lib.acct_fa_mask_bits_bytes(ctypes.byref(p)) == 0
+    p2.mask_bits = 4096
+    assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p2)) == 0
+    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p2)) == 2 * (2 * 2 * 128 * 4)
+    p2.mask_bits = 4096 + 64
+    assert lib.acct_fa_fwd(ctypes.byref(p2), addr, addr, None, 0, None) == -7     # misaligned buffer
+    p2.mask_bits = None
 
 
 def test_forward_rejects_misaligned_output_and_workspace():
@@ -206,6 +216,20 @@ def test_mask_classification():
     S = 256
     f16 = torch.float16
     tri = torch.triu(torch.ones(1, S, S, dtype=f16), 1)
+    # by default a mask tensor goes to the library as it is (its pre-pass finds the causal diagonal on the device)
+    assert not impl.DETECT_CAUSAL_MASKS
+    kind, m = impl._classify_mask(tri, S, S, f16)
+    assert kind == _capi.MASK_DENSE_F16 and m.data_ptr() == tri.data_ptr()
+    tile0 = torch.triu(torch.ones(1, 128, 128, dtype=f16), 1)
+    assert impl._classify_mask(tile0, S, S, f16)[0] == _capi.MASK_TILE_F16
+    impl.DETECT_CAUSAL_MASKS = True                      # opt-in: one device compare and host sync per mask tensor
+    try:
+        _test_mask_classification_with_detection(S, f16, tri)
+    finally:
+        impl.DETECT_CAUSAL_MASKS = False
+
+
+def _test_mask_classification_with_detection(S, f16, tri):
     assert impl._classify_mask(tri, S, S, f16)[0] == _capi.MASK_CAUSAL
     pad = torch.zeros(2, S, S, dtype=torch.uint8); pad[:, :, 200:] = 1
     kind, m8 = impl._classify_mask(pad, S, S, f16)
