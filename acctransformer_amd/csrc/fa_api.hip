@@ -191,22 +191,11 @@ acct::FaArgs make_args(const acct_fa_params* p) {
   return a;
 }
 
-// block classes of a dense mask (one byte per 128x128 block), then the scratch of the classification
-// pre-pass (16 bytes per block)
-size_t class_bytes(const acct_fa_params* p) {
-  if (!mask_is_dense(p)) return 0;
-  const size_t MB = p->mask_stride_b ? p->B : 1;
-  return align_up(MB * (size_t)((p->Sq + 127) / 128) * (size_t)((p->Sk + 127) / 128), 256);
-}
+// block classes of a dense mask: one byte per 128x128 block
 size_t flag_bytes(const acct_fa_params* p) {
   if (!mask_is_dense(p)) return 0;
   const size_t MB = p->mask_stride_b ? p->B : 1;
-  return class_bytes(p) + align_up(16 * MB * (size_t)((p->Sq + 127) / 128) * (size_t)((p->Sk + 127) / 128), 256);
-}
-// classify the blocks of a dense mask; fills a.blkflags (`flags`: flag_bytes(p) bytes)
-hipError_t prepare_mask(acct::FaArgs& a, const acct_fa_params* p, uint8_t* flags, hipStream_t st) {
-  a.blkflags = flags;
-  return acct::launch_mask_blocks(a, flags, (uint32_t*)(flags + class_bytes(p)), p->mask_stride_b ? p->B : 1, st);
+  return align_up(MB * (size_t)((p->Sq + 127) / 128) * (size_t)((p->Sk + 127) / 128), 256);
 }
 
 // per-key-column bitmaps of the mixed blocks of a dense mask (backward only): 16 bytes per (q block, key)
@@ -243,14 +232,9 @@ int mask_prepass(acct::FaArgs& a, const acct_fa_params* p, uint8_t* own, bool wa
   if (mask_is_dense(p)) a.blkflags = flags;
   if (cols) a.colbits = cbits;
   if (filled) return ACCT_OK;
-  if (mask_is_dense(p)) {
-    hipError_t e = prepare_mask(a, p, flags, st);
-    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask block kernel: %s", hipGetErrorString(e));
-  }
-  if (cols) {
-    hipError_t e = acct::launch_mask_colbits(a, flags, cbits, p->mask_stride_b ? p->B : 1, st);
-    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask bitmap kernel: %s", hipGetErrorString(e));
-  }
+  hipError_t e = mask_is_dense(p) ? acct::launch_mask_blocks(a, flags, cols ? cbits : nullptr, p->mask_stride_b ? p->B : 1, st)
+                                  : (cols ? acct::launch_mask_colbits(a, flags, cbits, 1, st) : hipSuccess);
+  if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "mask pre-pass kernel: %s", hipGetErrorString(e));
   return ACCT_OK;
 }
 

@@ -31,7 +31,7 @@ ACCT_DEV typename Elem<T>::V8 pack8(const float* x) {
 // dQ kernel (and delta): query-tile owner, structure of the forward kernel
 // ============================================================================
 template <typename T, int D, int QG, int NW, bool BIAS, bool DROP, bool MASKT>
-__global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
+ACCT_DEV void fa_bwd_dq_body(const FaArgs& a) {
   using E = Elem<T>;
   using V8 = typename E::V8;
   using C = SwzCfg<D>;
@@ -66,18 +66,28 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   const bool causal = a.mask_kind == kMaskCausal;
   if (causal) j_hi = min(j_hi, (q_end - 1) / 64);
   if (a.row_prefix) j_hi = min(j_hi, (((q_end - 1) / a.row_prefix + 1) * a.row_prefix - 1) / 64);
+  const int wqb = wq0 / 128;
+  BlkClassWindow flwin;                                     // block classes of a dense mask: 64 blocks at a time in scalar registers
+  bool flwin_ready = false;
   if (MASKT && a.mask_kind == kMaskDense) {
     // tiles at either end whose 128x128 blocks are wholly masked for every row block of this workgroup are
-    // not streamed at all (key padding: the padded tail of every sequence)
+    // not streamed at all (key padding: the padded tail of every sequence).  With at most 64 blocks in the
+    // band, one round trip to memory yields both the trimmed range and the wave's class window.
     const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc;
-    auto dead = [&](int j) {
-      for (int qb = qb_lo; qb <= qb_hi; qb++)
-        if (fl[(int64_t)qb * a.Tc + (j >> 1)] != kBlkSkip) return false;
-      return true;
-    };
-    trim_dead_tiles(j_lo, j_hi, lane, dead);
+    int b_lo = j_lo >> 1, b_hi = j_hi >> 1;
+    if (j_lo <= j_hi && flwin.init_trimmed(fl, 1, a.Tc, qb_lo, qb_hi - qb_lo + 1, min(wqb, qb_hi), b_lo, b_hi, lane)) {
+      j_lo = max(j_lo, b_lo * 2);
+      j_hi = min(j_hi, b_hi * 2 + 1);
+      flwin_ready = true;
+    } else {
+      auto dead = [&](int j) {
+        for (int qb = qb_lo; qb <= qb_hi; qb++)
+          if (fl[(int64_t)qb * a.Tc + (j >> 1)] != kBlkSkip) return false;
+        return true;
+      };
+      trim_dead_tiles(j_lo, j_hi, lane, dead);
+    }
   }
-  const int wqb = wq0 / 128;
   const int wkv_limit = a.row_prefix ? (wq0 / a.row_prefix + 1) * a.row_prefix : 0x7fffffff;
 
   // Q and dO fragments (B operands), delta and L of the lane's query row
@@ -173,8 +183,7 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
 
     // block classes of a dense mask: 64 blocks at a time into scalar registers
     const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
-    BlkClassWindow flwin;
-    flwin.init(flrow, 1, j_lo >> 1, j_hi >> 1, lane);
+    if (!flwin_ready) flwin.init(flrow, 1, j_lo >> 1, j_hi >> 1, lane);
     for (int j = j_lo; j <= j_hi; j++) {
       const uint32_t fl_cur = flwin.get(j >> 1, lane);
       const int buf = (j - j_lo) & 1;
@@ -419,6 +428,31 @@ __global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
   }
 }
 
+// The variant that knows mask tensors but neither a bias nor dropout carries a second body: a workgroup whose
+// rows see nothing but the causal pattern in a dense mask (block classes: clean before the diagonal, the
+// causal diagonal, skipped after it) runs the code of the variant without side inputs, by index compare.
+template <typename T, int D, int QG, int NW, bool BIAS, bool DROP, bool MASKT>
+__global__ void __launch_bounds__(64 * NW) fa_bwd_dq_kernel(const FaArgs a) {
+  if constexpr (MASKT && !BIAS && !DROP) {
+    if (a.mask_kind == kMaskDense) {
+      constexpr int BM = 32 * QG * NW;
+      int bh, rank;
+      wg_map(blockIdx.x, a.B * a.N, a.n_tiles, bh, rank);
+      const int q0 = (a.n_tiles - 1 - rank) * BM, q_end = min(q0 + BM, a.Sq);
+      const int qb_lo = q0 / 128, qb_hi = (q_end - 1) / 128;
+      const int kvb_lo = max(0, qb_lo - a.prev_blk), kvb_hi = min(a.Tc - 1, qb_hi + a.next_blk);
+      const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? bh / a.N : 0) * a.Tr) * a.Tc;
+      if (dense_lines_are_causal(fl, 1, a.Tc, qb_lo, qb_hi - qb_lo + 1, kvb_lo, kvb_hi, false, a, threadIdx.x & 63)) {
+        FaArgs c = a;
+        c.mask_kind = kMaskCausal;
+        fa_bwd_dq_body<T, D, QG, NW, false, false, false>(c);
+        return;
+      }
+    }
+  }
+  fa_bwd_dq_body<T, D, QG, NW, BIAS, DROP, MASKT>(a);
+}
+
 // Epilogue of the dK/dV kernel: dV (V role) or dK (K role) of a wave's key rows, scaled, converted and transposed
 // through the wave's own LDS region so that the global stores are whole rows.  acc[gk][db] = [d rows of block db,
 // key column l32] of key group gk; wk0 = first key row of the wave's pair.
@@ -518,7 +552,7 @@ template <int D> constexpr int dkdv_groups() { return D > 128 ? 1 : 2; }
 // MASKT = false compiles the mask-tensor handling out (no mask, or the causal mask by index compare):
 // the hot variant must not carry that code's register pressure.
 template <typename T, int D, bool BIAS, bool DROP, bool MASKT, int NGK = 2>
-__global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
+ACCT_DEV void fa_bwd_dkdv_body(const FaArgs& a) {
   static_assert(NGK == 2 || (NGK == 1 && !BIAS && !DROP), "one key group per wave: the plain variants only");
   using E = Elem<T>;
   using V8 = typename E::V8;
@@ -566,18 +600,28 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
     i_lo = max(i_lo, slice * per);
     i_hi = min(i_hi, (slice + 1) * per - 1);
   }
+  const int wkb = wk0 / 128;
+  BlkClassWindow flwin;                               // block classes of a dense mask: 64 blocks at a time in scalar registers
+  bool flwin_ready = false;
   if (MASKT && a.mask_kind == kMaskDense) {
     // query tiles at either end whose blocks are wholly masked for every key block of this workgroup are
-    // not streamed at all (key padding: a workgroup of padded keys has nothing to do)
+    // not streamed at all (key padding: a workgroup of padded keys has nothing to do).  With at most 64 query
+    // blocks, one round trip to memory yields both the trimmed range and the pair's class window.
     const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc;
-    auto dead = [&](int i) {
-      for (int kb = kb_lo; kb <= kb_hi; kb++)
-        if (fl[(int64_t)(i >> 1) * a.Tc + kb] != kBlkSkip) return false;
-      return true;
-    };
-    trim_dead_tiles(i_lo, i_hi, lane, dead);
+    int b_lo = i_lo >> 1, b_hi = i_hi >> 1;
+    if (i_lo <= i_hi && flwin.init_trimmed(fl, a.Tc, 1, kb_lo, kb_hi - kb_lo + 1, min(wkb, kb_hi), b_lo, b_hi, lane)) {
+      i_lo = max(i_lo, b_lo * 2);
+      i_hi = min(i_hi, b_hi * 2 + 1);
+      flwin_ready = true;
+    } else {
+      auto dead = [&](int i) {
+        for (int kb = kb_lo; kb <= kb_hi; kb++)
+          if (fl[(int64_t)(i >> 1) * a.Tc + kb] != kBlkSkip) return false;
+        return true;
+      };
+      trim_dead_tiles(i_lo, i_hi, lane, dead);
+    }
   }
-  const int wkb = wk0 / 128;
 
   // stationary B operands: K fragments (V role) or V fragments (K role) of the pair's 64 key rows;
   // lane holds key row 32 gk + l32, d = 16t + 8g ..
@@ -720,8 +764,7 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
       for (int t = 0; t < 4; t++) foff4_kept[t] = l32 * C::PITCH + swz_off(2 * t + g, C::swz(l32));
     }
     const uint8_t* flcol = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + (int64_t)mb * a.Tr * a.Tc + wkb : nullptr;
-    BlkClassWindow flwin;
-    flwin.init_descending(flcol, a.Tc, c_lo >> 2, c_hi >> 2, lane);
+    if (!flwin_ready) flwin.init_descending(flcol, a.Tc, c_lo >> 2, c_hi >> 2, lane);
     for (int n = 0; n <= npos; n++) {
       if ((n & 1) && (n >> 1) + 1 < ntile) stage(i_hi - ((n >> 1) + 1), smem + ((((n >> 1) + 1) & 1) * STAGEB));
       const int cpos = __builtin_amdgcn_readfirstlane(krole ? n - 1 : n);   // position of the chunk this wave works on in this step (wave-uniform: scalar)
@@ -959,6 +1002,33 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 
 #undef FOFF
 #undef TOFF
+
+// (two bodies in the variant that knows mask tensors only, as in the dQ kernel: a workgroup whose key blocks
+// see nothing but the causal pattern runs the code of the variant without side inputs)
+template <typename T, int D, bool BIAS, bool DROP, bool MASKT, int NGK = 2>
+__global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
+  if constexpr (MASKT && !BIAS && !DROP) {
+    if (a.mask_kind == kMaskDense) {
+      constexpr int BNK = 4 * 32 * NGK;
+      const int BH = a.B * a.N, n_wg = BH * a.n_tiles;
+      int wg = blockIdx.x;
+      if (a.q_split > 1) wg -= (wg / n_wg) * n_wg;
+      int bh, kt;
+      wg_map(wg, BH, a.n_tiles, bh, kt);
+      const int k0 = kt * BNK, k_end = min(k0 + BNK, a.Sk);
+      const int kb_lo = k0 / 128, kb_hi = (k_end - 1) / 128;
+      const int qb_lo = max(0, kb_lo - a.next_blk), qb_hi = min(a.Tr - 1, kb_hi + a.prev_blk);
+      const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? bh / a.N : 0) * a.Tr) * a.Tc;
+      if (dense_lines_are_causal(fl, a.Tc, 1, kb_lo, kb_hi - kb_lo + 1, qb_lo, qb_hi, true, a, threadIdx.x & 63)) {
+        FaArgs c = a;
+        c.mask_kind = kMaskCausal;
+        fa_bwd_dkdv_body<T, D, false, false, false, NGK>(c);
+        return;
+      }
+    }
+  }
+  fa_bwd_dkdv_body<T, D, BIAS, DROP, MASKT, NGK>(a);
+}
 
 // ---- launchers ----------------------------------------------------------------
 template <typename T, int D, bool BIAS, bool DROP>

@@ -197,6 +197,30 @@ struct BlkClassWindow {
     p = p_; stride = stride_; first = first_; last = last_;
     load(max(first_, last_ - 63), lane);
   }
+  // The window of the blocks [lo, hi] of line `own` and, in the same round trip to memory, the part of [lo, hi]
+  // that is not 'skip' in every one of the `n` lines line0 .. line0 + n - 1 (the row or column blocks a
+  // workgroup covers; line l, block x sits at tbl[l * line_step + x * stride]): lo and hi shrink to it (lo > hi
+  // when nothing is left).  For at most 64 blocks; returns false, with nothing done, when there are more.
+  ACCT_DEV bool init_trimmed(const uint8_t* tbl, int64_t stride_, int64_t line_step, int line0, int n, int own, int& lo, int& hi, int lane) {
+    if (hi - lo >= 64 || n > 2) return false;
+    p = tbl + (int64_t)own * line_step; stride = stride_; first = lo; last = hi; base = lo;
+    const int blk = lo + lane;
+    const bool in = blk <= hi;
+    // (all loads are issued before the first ballot waits for one)
+    const uint32_t f0 = in ? tbl[(int64_t)line0 * line_step + blk * stride_] : (uint32_t)kBlkSkip;
+    const uint32_t f1 = (in && n > 1) ? tbl[(int64_t)(line0 + 1) * line_step + blk * stride_] : (uint32_t)kBlkSkip;
+    const uint32_t fo = own == line0 ? f0 : (own == line0 + 1 && n > 1 ? f1 : (in ? p[blk * stride_] : 0u));
+    const uint64_t live = __ballot(in && !(f0 == kBlkSkip && f1 == kBlkSkip));
+    b0 = __ballot(in && (fo & 1u));
+    b1 = __ballot(in && (fo & 2u));
+    if (live) {
+      hi = lo + 63 - __builtin_clzll(live);
+      lo += __builtin_ctzll(live);
+    } else {
+      hi = lo - 1;
+    }
+    return true;
+  }
   ACCT_DEV void load(int first, int lane) {
     base = first;
     const int blk = first + lane;
@@ -211,6 +235,33 @@ struct BlkClassWindow {
     return (uint32_t)((b0 >> sh) & 1u) | ((uint32_t)((b1 >> sh) & 1u) << 1);
   }
 };
+
+// True when the block classes of a dense mask say that, inside the band, the `n` (<= 2) lines line0 .. of the class
+// table that a workgroup covers hold exactly the causal pattern: clean before the diagonal, the causal diagonal
+// class on it, skipped after it.  Such a workgroup gives the same results by index compare alone, with the code
+// that knows no mask tensor.  `lines_are_keys`: the lines are key blocks and the walk [lo, hi] runs over query
+// blocks (the dK/dV kernel); else the lines are query blocks and the walk runs over key blocks.  Element
+// (line l, block x) sits at tbl[l * line_step + x * stride].  At most 64 blocks are looked at (one load per
+// lane and line); more give false.  Every wave of the workgroup arrives at the same answer.
+ACCT_DEV bool dense_lines_are_causal(const uint8_t* tbl, int64_t stride, int64_t line_step, int line0, int n, int lo, int hi,
+                                     bool lines_are_keys, const FaArgs& a, int lane) {
+  if (hi - lo >= 64 || n > 2 || lo > hi) return false;
+  const int blk = lo + lane;
+  bool ok = true;
+  uint32_t f[2];
+#pragma unroll
+  for (int l = 0; l < 2; l++) f[l] = (l < n && blk <= hi) ? tbl[(int64_t)(line0 + l) * line_step + blk * stride] : 0u;
+#pragma unroll
+  for (int l = 0; l < 2; l++)
+    if (l < n && blk <= hi) {
+      const int qb = lines_are_keys ? blk : line0 + l, kb = lines_are_keys ? line0 + l : blk;
+      bool in_band = (kb - a.next_blk <= qb) && (qb <= kb + a.prev_blk);
+      if (a.row_prefix) in_band = in_band && kb <= ((qb * 128 / a.row_prefix + 1) * a.row_prefix - 1) / 128;
+      const uint32_t want = kb < qb ? (uint32_t)kBlkClean : (kb == qb ? (uint32_t)kBlkTriu : (uint32_t)kBlkSkip);
+      ok = ok && (!in_band || f[l] == want);
+    }
+  return __all(ok);
+}
 
 // four consecutive mask / dropout bytes starting at column kv of a row
 ACCT_DEV uint32_t load_u8x4(const uint8_t* row, int kv, int limit, bool vec_ok) {

@@ -19,7 +19,7 @@
 namespace acct {
 
 template <typename T, int D, int QG, int NW, bool BIAS, bool DROP, bool MASKT, int KT = 2>
-__global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
+ACCT_DEV void fa_fwd_body(const FaArgs& a) {
   static_assert(KT == 2 || KT == 4, "key tiles are 64 or 128 rows (with a bias, 128 rows take the key-only form of it only)");
   constexpr int BN = 32 * KT;                       // key rows per tile
   constexpr int FRING = 4, VRING = 3;   // fragment reads in flight ahead of their MFMA (K row-major / V transposed)
@@ -55,18 +55,28 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   const bool causal = a.mask_kind == kMaskCausal;
   if (causal) j_hi = min(j_hi, (q_end - 1) / BN);
   if (a.row_prefix) j_hi = min(j_hi, (((q_end - 1) / a.row_prefix + 1) * a.row_prefix - 1) / BN);
+  const int wqb = wq0 / 128;                                // 128-block of this wave's rows
+  BlkClassWindow flwin;                                     // block classes of a dense mask: 64 blocks at a time in scalar registers
+  bool flwin_ready = false;
   if (MASKT && a.mask_kind == kMaskDense) {
     // tiles at either end whose 128x128 blocks are wholly masked for every row block of this workgroup are
-    // not streamed at all (key padding: the padded tail of every sequence)
+    // not streamed at all (key padding: the padded tail of every sequence).  With at most 64 blocks in the
+    // band, one round trip to memory yields both the trimmed range and the wave's class window.
     const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc;
-    auto dead = [&](int j) {
-      for (int qb = qb_lo; qb <= qb_hi; qb++)
-        if (fl[(int64_t)qb * a.Tc + j / TPB] != kBlkSkip) return false;
-      return true;
-    };
-    trim_dead_tiles(j_lo, j_hi, lane, dead);
+    int b_lo = j_lo / TPB, b_hi = j_hi / TPB;
+    if (j_lo <= j_hi && flwin.init_trimmed(fl, 1, a.Tc, qb_lo, qb_hi - qb_lo + 1, min(wqb, qb_hi), b_lo, b_hi, lane)) {
+      j_lo = max(j_lo, b_lo * TPB);
+      j_hi = min(j_hi, b_hi * TPB + TPB - 1);
+      flwin_ready = true;
+    } else {
+      auto dead = [&](int j) {
+        for (int qb = qb_lo; qb <= qb_hi; qb++)
+          if (fl[(int64_t)qb * a.Tc + j / TPB] != kBlkSkip) return false;
+        return true;
+      };
+      trim_dead_tiles(j_lo, j_hi, lane, dead);
+    }
   }
-  const int wqb = wq0 / 128;                                // 128-block of this wave's rows
   const int wkv_limit = a.row_prefix ? (wq0 / a.row_prefix + 1) * a.row_prefix : 0x7fffffff;   // keys past it are absent
 
   // ---- Q fragments (B operand of K Q^T): lane holds row l32, d = 16t + 8g .. +7 ----
@@ -155,8 +165,7 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   ACCT_LDS char* drop_lds = smem + 4 * TILEB + NW * BIASB + wave * (2 * DropStage::BYTES);
   // ---- the phases of a tile step: classification, S^T = K Q^T, online softmax, O^T += V^T P^T ----
   const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
-  BlkClassWindow flwin;                                      // block classes of a dense mask: 64 blocks at a time in scalar registers
-  if (j_lo <= j_hi) flwin.init(flrow, 1, j_lo / TPB, j_hi / TPB, lane);
+  if (!flwin_ready && j_lo <= j_hi) flwin.init(flrow, 1, j_lo / TPB, j_hi / TPB, lane);
   enum : uint32_t { kAct = 1u, kApply = 2u, kDiag = 4u };
   // what this wave does with tile j (tiles must be asked for in ascending order)
   auto classify = [&](int j) -> uint32_t {
@@ -451,6 +460,32 @@ __global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
   }
 }
 
+
+// The variant that knows mask tensors but neither a bias nor dropout carries a second body: a workgroup whose
+// rows see nothing but the causal pattern in a dense mask (block classes: clean before the diagonal, the
+// causal diagonal, skipped after it) runs the code of the variant without side inputs, by index compare.
+// A causal mask given as a tensor then costs one look at the class table per workgroup.
+template <typename T, int D, int QG, int NW, bool BIAS, bool DROP, bool MASKT, int KT = 2>
+__global__ void __launch_bounds__(64 * NW) fa_fwd_kernel(const FaArgs a) {
+  if constexpr (MASKT && !BIAS && !DROP) {
+    if (a.mask_kind == kMaskDense) {
+      constexpr int BM = 32 * QG * NW;
+      int bh, rank;
+      wg_map(blockIdx.x, a.B * a.N, a.n_tiles, bh, rank);
+      const int q0 = (a.n_tiles - 1 - rank) * BM, q_end = min(q0 + BM, a.Sq);
+      const int qb_lo = q0 / 128, qb_hi = (q_end - 1) / 128;
+      const int kvb_lo = max(0, qb_lo - a.prev_blk), kvb_hi = min(a.Tc - 1, qb_hi + a.next_blk);
+      const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? bh / a.N : 0) * a.Tr) * a.Tc;
+      if (dense_lines_are_causal(fl, 1, a.Tc, qb_lo, qb_hi - qb_lo + 1, kvb_lo, kvb_hi, false, a, threadIdx.x & 63)) {
+        FaArgs c = a;
+        c.mask_kind = kMaskCausal;
+        fa_fwd_body<T, D, QG, NW, false, false, false, KT>(c);
+        return;
+      }
+    }
+  }
+  fa_fwd_body<T, D, QG, NW, BIAS, DROP, MASKT, KT>(a);
+}
 
 template <typename T, int D, int QG, int NW, bool BIAS, bool DROP, int KT>
 static hipError_t launch_fwd_kt(FaArgs a, hipStream_t st) {

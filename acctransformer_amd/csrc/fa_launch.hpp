@@ -59,14 +59,14 @@ hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t
 // false when the kernel translation units were compiled with a reduced variant set (ACCT_DEV_BUILD)
 bool launch_variants_complete();
 
-// classify the 128x128 blocks of a dense mask into clean / apply / skip / causal diagonal; `scan` is scratch of
-// 16 bytes per block (per-row "has an unmasked element" bits between the two launches of the fast path)
-hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, uint32_t* scan, int MB, hipStream_t st);
+// classify the 128x128 blocks of a dense mask into clean / apply / skip / causal diagonal and, with `colbits`
+// non-null, pack its 'apply' blocks into per-key-column bitmaps [MB, Tr, Sk, 4 x u32] (one launch for aligned masks)
+hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, uint32_t* colbits, int MB, hipStream_t st);
 // pack the dropout mask into keep bits by query row [B*N, Sq, droprow_w] and / or by key column [B*N, Tr, Sk, 4]
 hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st);
 // the same two bitmaps generated from (a.philox_k0, a.philox_k1, a.philox_offset, a.philox_thr) instead of read from a mask
 hipError_t launch_drop_philox(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st);
-// pack the 'apply' blocks of a dense mask into per-key-column bitmaps [MB, Tr, Sk, 4 x u32]
+// the column bitmaps by themselves (and the compact tile's: out[key][4])
 hipError_t launch_mask_colbits(const FaArgs& a, const uint8_t* flags, uint32_t* out, int MB, hipStream_t st);
 
 }  // namespace acct

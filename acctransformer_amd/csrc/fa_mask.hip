@@ -18,19 +18,23 @@ namespace acct {
 
 constexpr uint8_t kBlkAllMasked = 255;  // provisional: resolved to skip or apply below
 
-// Fast path (Sk and the mask pointers 16-byte aligned), in two launches so that the work spreads over the
-// chip whatever the shape (a [1, 2048, 2048] mask has 16 row blocks but 256 blocks):
+// Fast path (Sk and the mask pointers 16-byte aligned): ONE launch that leaves the block classes and, for the
+// dK/dV kernel, the column bitmaps of the mixed blocks (every launch costs a few microseconds of a step that
+// takes a few hundred).  One workgroup of 256 threads per (mask batch, q block, key block) inside the band, so
+// that the work spreads over the chip whatever the shape (a [1, 2048, 2048] mask has 16 row blocks but 256
+// blocks).  Thread t owns 64 consecutive elements of row t % 128 (half t / 128 of the block's 128 columns),
+// four or eight 16-byte loads, as a 64-bit "nonzero" mask.
 //
-// fa_mask_scan_kernel: one workgroup of 256 threads per (mask batch, q block, key block) inside the band.
-// Thread t owns 64 consecutive elements of row t % 128 (half t / 128 of the block's 128 columns), four or
-// eight 16-byte loads.  It leaves the block's provisional class (clean / apply / all masked / the causal
-// diagonal pattern) and, per row, whether the row has an unmasked element in this block (128 bits).
-//
-// fa_mask_resolve_kernel: one wave per (mask batch, q block) ORs those row bits over the band and turns
-// "all masked" into skip when every row of the q block has an unmasked key somewhere, else into apply.
+// A wholly masked block may be skipped only if every row of its q block sees an unmasked key somewhere (see the
+// top of the file).  A workgroup cannot see the other blocks of its row block's band, so it checks a sufficient
+// condition on two of them that it reads itself: every row has an unmasked key in the first block of the band
+// or in the diagonal block.  That holds for causal, banded, prefix and document masks (the diagonal entry is
+// visible) and for key padding (the first keys are); where it fails although the rows do see keys elsewhere,
+// the block is classed 'apply' instead of 'skip', which gives the same results bit for bit, only slower.
 template <int ES>
-__global__ void __launch_bounds__(256) fa_mask_scan_kernel(const FaArgs a, uint8_t* flags, uint32_t* rowseen) {
-  __shared__ unsigned long long s_seen[2];
+__global__ void __launch_bounds__(256) fa_mask_prepass_kernel(const FaArgs a, uint8_t* flags, uint32_t* colbits) {
+  __shared__ unsigned long long s_bits[128][2];         // nonzero bits of the block: [row][column half]
+  __shared__ unsigned long long s_seen[2];              // rows (bit = row % 64) with an unmasked key in the blocks probed
   const int kvb = blockIdx.x % a.Tc, qb = (blockIdx.x / a.Tc) % a.Tr, mb = blockIdx.x / (a.Tc * a.Tr);
   const int tid = threadIdx.x;
   int lo = max(0, qb - a.prev_blk), hi = min(a.Tc - 1, qb + a.next_blk);
@@ -40,84 +44,86 @@ __global__ void __launch_bounds__(256) fa_mask_scan_kernel(const FaArgs a, uint8
     if (tid == 0) flags[blk] = kBlkClean;
     return;
   }
-  if (tid < 2) s_seen[tid] = 0;
-  __syncthreads();
   const int rib = tid & 127, half = tid >> 7, row = qb * 128 + rib, c0 = half * 64;
   const uint8_t* mrow = a.mask + ((int64_t)mb * a.mask_sb + (int64_t)min(row, a.Sq - 1) * a.Sk) * ES;
-  const bool on_diag = kvb == qb;                       // the per-element pattern matters on the diagonal block only
-  bool has_zero = false, has_nonzero = false, tri_bad = false;
-  if (row < a.Sq) {
+  // this thread's 64 elements of key block kb: nz = nonzero bits, valid = bits of the elements that exist
+  auto scan = [&](int kb, unsigned long long& nz, unsigned long long& valid) {
+    nz = 0; valid = 0;
+    if (row >= a.Sq) return;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      const int col = c0 + 16 * i, kv = kvb * 128 + col;
+      const int kv = kb * 128 + c0 + 16 * i;
       if (kv < a.Sk) {                                  // Sk % 16 == 0: a piece is entirely inside or outside
-        uint32_t nz = 0;                                // bit e: element e of these 16 is nonzero
+        uint32_t bits = 0;                              // bit e: element e of these 16 is nonzero
 #pragma unroll
         for (int h = 0; h < ES; h++) {
           const u32x4 v = *reinterpret_cast<const u32x4*>(mrow + (int64_t)kv * ES + 16 * h);
 #pragma unroll
           for (int w = 0; w < 4; w++) {
             if (ES == 1) {
-              // a byte is zero iff (x - 0x01010101) & ~x & 0x80808080 has its top bit set
-              has_nonzero |= v[w] != 0;
-              has_zero |= ((v[w] - 0x01010101u) & ~v[w] & 0x80808080u) != 0;
-              if (on_diag) {
 #pragma unroll
-                for (int e = 0; e < 4; e++) nz |= (((v[w] >> (8 * e)) & 0xffu) != 0 ? 1u : 0u) << (4 * w + e);
-              }
+              for (int e = 0; e < 4; e++) bits |= (((v[w] >> (8 * e)) & 0xffu) != 0 ? 1u : 0u) << (4 * w + e);
             } else {
               // 2-byte floating-point elements: the sign of a zero does not count
-              const uint32_t lo16 = v[w] & 0x7fffu, hi16 = (v[w] >> 16) & 0x7fffu;
-              has_nonzero |= (lo16 | hi16) != 0;
-              has_zero |= lo16 == 0 || hi16 == 0;
-              if (on_diag) nz |= ((lo16 != 0 ? 1u : 0u) | (hi16 != 0 ? 2u : 0u)) << (8 * h + 2 * w);
+              bits |= (((v[w] & 0x7fffu) != 0 ? 1u : 0u) | (((v[w] >> 16) & 0x7fffu) != 0 ? 2u : 0u)) << (8 * h + 2 * w);
             }
           }
         }
-        if (on_diag) {
+        nz |= (unsigned long long)bits << (16 * i);
+        valid |= 0xffffull << (16 * i);
+      }
+    }
+  };
+  unsigned long long nz, valid;
+  scan(kvb, nz, valid);
+  // the causal pattern on the diagonal block: column c0 + e is masked iff it comes after row rib
+  const int d = rib - c0;                               // columns above bit d are "after the row"
+  const unsigned long long tri = d < 0 ? ~0ull : (d >= 63 ? 0ull : (~0ull << (d + 1)));
+  const bool on_diag = kvb == qb;
+  const int any_m = __syncthreads_or(nz != 0), any_u = __syncthreads_or((~nz & valid) != 0);
+  const int bad = __syncthreads_or(on_diag && ((nz ^ tri) & valid) != 0);
+  uint8_t cls = !any_m ? kBlkClean : (any_u ? ((on_diag && !bad) ? kBlkTriu : kBlkApply) : kBlkSkip);
+  if (cls == kBlkSkip) {                                // (uniform: the whole workgroup takes the branch)
+    if (tid < 2) s_seen[tid] = 0;
+    __syncthreads();
+    const int probe[2] = {lo, (qb >= lo && qb <= hi && qb != lo) ? qb : -1};
 #pragma unroll
-          for (int e = 0; e < 16; e++) tri_bad |= (((nz >> e) & 1u) != 0) != (col + e > rib);
-        }
+    for (int k = 0; k < 2; k++)
+      if (probe[k] >= 0 && probe[k] != kvb) {
+        unsigned long long pnz, pvalid;
+        scan(probe[k], pnz, pvalid);
+        const unsigned long long seen = __ballot((~pnz & pvalid) != 0);
+        if ((tid & 63) == 0 && seen) atomicOr(&s_seen[(tid >> 6) & 1], seen);
+      }
+    __syncthreads();
+    const int nrow = min(128, a.Sq - qb * 128);         // rows past Sq do not count
+    bool ok = true;
+#pragma unroll
+    for (int w = 0; w < 2; w++) {
+      const int n = min(64, max(0, nrow - 64 * w));
+      const unsigned long long need = n >= 64 ? ~0ull : ((1ull << n) - 1ull);
+      ok = ok && (s_seen[w] & need) == need;
+    }
+    if (!ok) cls = kBlkApply;
+  }
+  if (tid == 0) flags[blk] = cls;
+  if (cls == kBlkApply && colbits) {
+    // the block packed by key column: 128 bits per key, bit r = mask[128 qb + r][key]
+    s_bits[rib][half] = nz;
+    __syncthreads();
+    const int col = tid & 127, kv = kvb * 128 + col;
+    if (kv < a.Sk) {
+      const ACCT_LDS uint32_t* sb = (const ACCT_LDS uint32_t*)&s_bits[0][0] + (col >> 5);   // the 32-bit piece that holds the column
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        const int i = 2 * half + j;
+        uint32_t w = 0;
+#pragma unroll 8
+        for (int r = 0; r < 32; r++) w |= ((sb[(32 * i + r) * 4] >> (col & 31)) & 1u) << r;
+        colbits[(((int64_t)mb * a.Tr + qb) * a.Sk + kv) * 4 + i] = w;
       }
     }
   }
-  // rows 64 (tid / 64 % 2) .. +63 of the block: one ballot per wave, the two column halves OR-ed in LDS
-  const unsigned long long seen = __ballot(has_zero);
-  if ((tid & 63) == 0) atomicOr(&s_seen[(tid >> 6) & 1], seen);
-  const int any_m = __syncthreads_or(has_nonzero), any_u = __syncthreads_or(has_zero), bad = __syncthreads_or(tri_bad);
-  if (tid < 4) rowseen[blk * 4 + tid] = (uint32_t)(s_seen[tid >> 1] >> (32 * (tid & 1)));
-  if (tid == 0) flags[blk] = !any_m ? kBlkClean : (!any_u ? kBlkAllMasked : ((on_diag && !bad) ? kBlkTriu : kBlkApply));
-}
-
-__global__ void __launch_bounds__(64) fa_mask_resolve_kernel(const FaArgs a, uint8_t* flags, const uint32_t* rowseen) {
-  const int qb = blockIdx.x % a.Tr, mb = blockIdx.x / a.Tr, lane = threadIdx.x;
-  int lo = max(0, qb - a.prev_blk), hi = min(a.Tc - 1, qb + a.next_blk);
-  if (a.row_prefix) hi = min(hi, ((qb * 128 / a.row_prefix + 1) * a.row_prefix - 1) / 128);
-  uint8_t* frow = flags + ((int64_t)mb * a.Tr + qb) * a.Tc;
-  const u32x4* seen = reinterpret_cast<const u32x4*>(rowseen) + ((int64_t)mb * a.Tr + qb) * a.Tc;
-  u32x4 acc = {0u, 0u, 0u, 0u};
-  bool any_allmasked = false;
-  for (int kvb = lo + lane; kvb <= hi; kvb += 64) {
-    const u32x4 v = seen[kvb];
-#pragma unroll
-    for (int w = 0; w < 4; w++) acc[w] |= v[w];
-    any_allmasked |= frow[kvb] == kBlkAllMasked;
-  }
-  if (!__any(any_allmasked)) return;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1)
-#pragma unroll
-    for (int w = 0; w < 4; w++) acc[w] |= (uint32_t)__shfl_xor((int)acc[w], off);
-  const int nrow = min(128, a.Sq - qb * 128);           // rows past Sq do not count
-  bool rows_ok = true;
-#pragma unroll
-  for (int w = 0; w < 4; w++) {
-    const int n = min(32, max(0, nrow - 32 * w));
-    const uint32_t need = n >= 32 ? 0xffffffffu : ((1u << n) - 1u);
-    rows_ok = rows_ok && (acc[w] & need) == need;
-  }
-  for (int kvb = lo + lane; kvb <= hi; kvb += 64)
-    if (frow[kvb] == kBlkAllMasked) frow[kvb] = rows_ok ? kBlkSkip : kBlkApply;
 }
 
 // Generic path (any alignment): one workgroup per (mask batch, q block); thread t scans 64 columns of row t/2
@@ -337,22 +343,25 @@ hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbit
   return hipGetLastError();
 }
 
-hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, uint32_t* scan, int MB, hipStream_t st) {
-  // fast path: every 16-element piece of a row is 16-byte aligned and entirely inside or outside the row
-  const bool vec = (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 15) == 0;
-  if (vec) {
+// true when launch_mask_blocks takes the fast path, which also writes the column bitmaps
+static bool mask_prepass_is_fused(const FaArgs& a) {
+  // every 16-element piece of a row is 16-byte aligned and entirely inside or outside the row
+  return (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 15) == 0;
+}
+
+hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, uint32_t* colbits, int MB, hipStream_t st) {
+  if (mask_prepass_is_fused(a)) {
     const dim3 grid((unsigned)((long long)MB * a.Tr * a.Tc));
-    if (a.mask_es == 2) hipLaunchKernelGGL(fa_mask_scan_kernel<2>, grid, dim3(256), 0, st, a, flags, scan);
-    else hipLaunchKernelGGL(fa_mask_scan_kernel<1>, grid, dim3(256), 0, st, a, flags, scan);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(fa_mask_resolve_kernel, dim3((unsigned)(MB * a.Tr)), dim3(64), 0, st, a, flags, (const uint32_t*)scan);
+    if (a.mask_es == 2) hipLaunchKernelGGL(fa_mask_prepass_kernel<2>, grid, dim3(256), 0, st, a, flags, colbits);
+    else hipLaunchKernelGGL(fa_mask_prepass_kernel<1>, grid, dim3(256), 0, st, a, flags, colbits);
     return hipGetLastError();
   }
   const dim3 grid((unsigned)(MB * a.Tr));
   if (a.mask_es == 2) hipLaunchKernelGGL(fa_mask_blocks_kernel<2>, grid, dim3(256), 0, st, a, flags);
   else hipLaunchKernelGGL(fa_mask_blocks_kernel<1>, grid, dim3(256), 0, st, a, flags);
-  return hipGetLastError();
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || !colbits) return e;
+  return launch_mask_colbits(a, flags, colbits, MB, st);
 }
 
 }  // namespace acct

@@ -87,16 +87,16 @@ def test_null_outputs_and_workspace_sizes():
     m = torch.zeros(1, 128, 128, dtype=torch.uint8)
     q = torch.zeros(2, 2, 128, 128, dtype=torch.float16)
     p2 = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m)
-    # block classes (padded to 256) and the classification pre-pass's scratch (16 bytes per block, padded)
-    assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p2)) == 256 + 256
+    # block classes (padded to 256)
+    assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p2)) == 256
     raw = (ctypes.c_char * 128)()
     addr = (ctypes.addressof(raw) + 63) // 64 * 64
     # backward without its workspace is refused before any launch
     assert lib.acct_fa_bwd(ctypes.byref(p2), *([addr] * 6), None, 0, None) == -7
-    # D and -LSE*log2e rows, block classes + scratch (padded to 256 each), key-column bitmaps: 16 bytes per (q block, key)
-    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p2)) == 2 * (2 * 2 * 128 * 4) + 512 + 1 * 1 * 128 * 16
-    # a caller-held mask_bits buffer takes the classes, the scratch and the bitmaps out of both workspaces
-    assert lib.acct_fa_mask_bits_bytes(ctypes.byref(p2)) == 512 + 128 * 16
+    # D and -LSE*log2e rows, block classes (padded to 256), key-column bitmaps: 16 bytes per (q block, key)
+    assert lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p2)) == 2 * (2 * 2 * 128 * 4) + 256 + 1 * 1 * 128 * 16
+    # a caller-held mask_bits buffer takes the classes and the bitmaps out of both workspaces
+    assert lib.acct_fa_mask_bits_bytes(ctypes.byref(p2)) == 256 + 128 * 16
     assert lib.acct_fa_mask_bits_bytes(ctypes.byref(p)) == 0
     p2.mask_bits = 4096
     assert lib.acct_fa_fwd_workspace_bytes(ctypes.byref(p2)) == 0
