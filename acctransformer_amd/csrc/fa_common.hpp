@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fa_index_math.hpp"
+
 namespace acct {
 
 typedef _Float16 f16;
@@ -140,24 +142,6 @@ struct FaArgs {
 
 enum : int { kMaskNone = 0, kMaskDense = 1, kMaskTile = 3, kMaskCausal = 4 };
 enum : uint8_t { kBlkClean = 0, kBlkApply = 1, kBlkSkip = 2, kBlkTriu = 3 };
-
-// Workgroup id -> (batch*head, launch rank of the tile; rank 0 is launched first).  Workgroups are
-// handed to the 8 XCDs round robin (id % 8), each XCD with its own L2.  With many heads the plain
-// "head fastest" order gives every CU of an XCD a different head and nothing is shared; instead the
-// heads of an XCD are taken 8 at a time and all tiles of those 8 heads are launched together, so
-// that the workgroups streaming the same K/V (or Q/dO) rows run side by side on one L2.
-ACCT_DEV void wg_map(int id, int BH, int n_tiles, int& bh, int& rank) {
-  if (BH > 64 && (BH & 63) == 0) {
-    const int xcd = id & 7, slot = id >> 3;
-    const int per_group = 8 * n_tiles;
-    const int grp = slot / per_group, r = slot - grp * per_group;
-    rank = r >> 3;
-    bh = xcd + 8 * (grp * 8 + (r & 7));
-  } else {
-    bh = id % BH;
-    rank = id / BH;
-  }
-}
 
 // Shrinks the tile range [lo, hi] from both ends while dead(tile) holds.  The 64 lanes of the wave test 64
 // tiles at a time (one round trip to memory per 64 tiles instead of one per tile); every wave of the
@@ -309,36 +293,8 @@ ACCT_DEV void load_bias4(const T* row, int kv, int limit, bool vec_ok, float out
 }
 
 // ---- swizzled LDS tiles filled by direct-to-LDS loads --------------------------
-// Row pitch is a power of two (no padding, as the DMA writes 64 consecutive 16-byte
-// slots per wave instruction); the 16-byte chunk c of row r lives in slot c ^ swz(r).
-// The LDS serves a 16-byte read in groups of 16 lanes over 64 four-byte banks, so the
-// fragment reads (lane = row) need the 16 rows of a group in 16 different slots of the
-// 256 bytes the banks span: measured 4.3 clocks per wave instruction against 8.2 when
-// only eight rows differ.  For 256-byte rows that is a four-bit swizzle,
-// swz(r) = ((r & 3) << 1) | ((r >> 2) & 1) | (r & 8); its low three bits also put one
-// 32-byte chunk PAIR of four consecutive rows into four different pairs of slots, which
-// is what the transposed 8-byte reads (4 rows x 32 bytes per 16 lanes) need.  For
-// 128-byte rows two consecutive rows span the banks and swz(r) = (r >> 1) & 7.
+// (the swizzle itself: SwzCfg in fa_index_math.hpp)
 #define ACCT_GLB __attribute__((address_space(1)))
-
-ACCT_DEV int swz3(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
-
-template <int D> struct SwzCfg {
-  static constexpr int KS = (D + 15) / 16;      // 16-wide k-steps across the head dim (the last one half empty when D % 16 == 8)
-  static constexpr int DB = (D + 31) / 32;      // 32-wide blocks across the head dim
-  static constexpr int CPR = D / 8;             // valid 16-byte chunks per row
-  static constexpr int CH = D <= 64 ? 8 : (D <= 128 ? 16 : 32);   // chunk slots per LDS row
-  static constexpr int PITCH = CH * 16;
-  static constexpr int RPI = 64 / CH;           // rows covered by one wave-wide DMA instruction
-  // (rows of 512 bytes wrap around the banks twice: the four-bit swizzle of the 256-byte rows serves them too)
-  static ACCT_DEV int swz(int row) { return CH >= 16 ? (swz3(row) | (row & 8)) : ((row >> 1) & 7); }
-  // Transposed reads come in pairs, rows r..r+3 and r+8..r+11 with r % 16 < 8: the second row group has
-  // the top swizzle bit set, so its slot differs in that bit.  Which way depends only on the 32-column
-  // block db the read belongs to (chunk 4 db + 0..3), i.e. the distance is a compile-time constant.
-  static constexpr int tr_hi(int db) {
-    return 8 * PITCH + (CH >= 16 ? (((db >> 1) & 1) ? -128 : 128) : ((db & 1) ? -64 : 64));
-  }
-};
 
 // Stage rows [row0, row0 + ROWS) of a row-major global matrix into a swizzled LDS
 // tile with NW waves.  Rows past nrows repeat the last valid row (finite data whose
@@ -518,12 +474,5 @@ struct DropRowStage {
   }
 };
 
-
-// idx / n for idx < 1024 and n <= 32 (the epilogues' chunk index -> row): exact with a 16-bit reciprocal
-ACCT_DEV int div_small(int idx, uint32_t inv16) { return (int)(((uint32_t)idx * inv16) >> 16); }
-ACCT_DEV uint32_t recip16(int n) { return (65536u + (uint32_t)n - 1u) / (uint32_t)n; }
-
-// byte offset of logical chunk `lc` in a row whose swz3(row) is `swz`
-ACCT_DEV int swz_off(int lc, int swz) { return (lc ^ swz) << 4; }
 
 }  // namespace acct

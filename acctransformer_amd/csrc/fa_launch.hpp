@@ -22,32 +22,6 @@ inline hipError_t allow_dynamic_lds(const void* kern, size_t bytes) {
   return e;
 }
 
-// The kernels are built for the head dims 40, 64, 80, 128, 160 and 256.  Any other multiple of 8 runs on the next
-// built size of its row layout (128-, 256- or 512-byte LDS rows): the columns past the head dim are never loaded
-// as operands (zero fragments) and never stored.
-inline int head_dim_class(int D) {
-  if (D == 40 || D == 80 || D == 160) return D;
-  return D <= 64 ? 64 : (D <= 128 ? 128 : 256);
-}
-
-// The dK/dV kernel gives every workgroup 256 keys (128 above head dim 128) of one head and all query rows.  With
-// few heads and a short key sequence (cross attention on 77 keys) that is a handful of workgroups for 256 CUs:
-// the query range is then cut into q_split slices that run side by side, and a second kernel adds their sums.
-// Returns q_split (1 = no split) and the bytes of workspace the slices' sums take.
-// `n_cu`: compute units of the device that runs the launch; the workspace-size query passes the 256 of a whole
-// MI355X, which is also the upper bound of what a partition of it asks for.
-struct DkdvSplit { int q_split; size_t part_bytes; };
-inline DkdvSplit dkdv_split(int B, int N, int Sq, int Sk, int D, int n_cu = 256) {
-  const int dc = head_dim_class(D), ngk = dc > 128 ? 1 : 2, db = (dc + 31) / 32;
-  const long long n_wg = (long long)B * N * ((Sk + 128 * ngk - 1) / (128 * ngk));
-  const long long tiles64 = (Sq + 63) / 64;
-  long long s = (n_cu > 256 ? 256 : n_cu) / n_wg;
-  if (tiles64 / 8 < s) s = tiles64 / 8;              // a slice keeps at least 512 query rows
-  if (s > 16) s = 16;
-  if (s < 2) return {1, 0};
-  return {(int)s, (size_t)s * (size_t)n_wg * 8 * ngk * db * 1024 * sizeof(float)};
-}
-
 // forward: variant 3 = 8 waves x 32 query rows, 1 = 4 waves x 32 rows; the bias / dropout
 // variants are picked from a.alibi / a.droprow
 hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st);

@@ -1027,6 +1027,45 @@ def test_inference_operator_at_its_length_limit():
     _gate(_np(orc.torch_unfused_fwd_fp32(q, k, v)), y, what="y at S = 8192")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Sq, Sk", [(512, 2048), (256, 16384)])
+def test_loss_scaled_upstream_gradient(dtype, Sq, Sk):
+    # fp16 training runs the backward on a loss-scaled dO (x 2^10 .. 2^15).  dS = P (dP - D) is packed to the I/O
+    # dtype before it feeds the dK / dQ products, as in the reference (its dS is fp16,
+    # flash_attention_bwd.py:161-181), so fp16 overflows where |dS| reaches 65504; above 4096 keys the kernels
+    # carry P with a factor 2^p_shift (one power of two per doubling of Sk: 2 at 16384 keys) and the bound is
+    # 65504 / 2^p_shift.  The test derives max |dS| from the fp64 operator and checks both sides of that bound:
+    # inside it the gradients of the scaled dO are the scaled gradients, to the gate; bf16 has no such bound.
+    D = 64
+    q, dO0 = _gen((1, 2, Sq, D), 301), _gen((1, 2, Sq, D), 304)
+    k, v = _gen((1, 2, Sk, D), 302), _gen((1, 2, Sk, D), 303)
+    scale = D ** -0.5
+    base = (dO0.float() * 2.0 ** -6).to(dtype)                    # the unscaled upstream gradient
+    qf, kf, vf, df = (_np(t).astype(np.float64) for t in (q.to(dtype), k.to(dtype), v.to(dtype), base))
+    sc = np.einsum("bhqd,bhkd->bhqk", qf, kf) * scale
+    P = np.exp(sc - sc.max(-1, keepdims=True)); P /= P.sum(-1, keepdims=True)
+    O = np.einsum("bhqk,bhkd->bhqd", P, vf)
+    dS = P * (np.einsum("bhqd,bhkd->bhqk", df, vf) - (df * O).sum(-1, keepdims=True))
+    ds_max = float(np.abs(dS).max())
+    shift = max(0, min(8, int(np.log2(Sk)) - 12))
+    tol = dict(atol=ATOL_BF16, rtol=RTOL_BF16) if dtype == torch.bfloat16 else dict(atol=ATOL, rtol=RTOL)
+    ref = orc.unfused_bwd(_np(q.to(dtype)), _np(k.to(dtype)), _np(v.to(dtype)), _np(base), scale=scale)
+    for lg in (10, 15):
+        c = 2.0 ** lg
+        assert c * ds_max * 2 ** shift < 0.5 * 65504, "the case is meant to lie inside the bound"
+        _, _, g = _run(q.to(dtype), k.to(dtype), v.to(dtype), (base.float() * c).to(dtype), scale=scale)
+        for name, r, got in zip(("dQ", "dK", "dV"), ref, g):
+            assert torch.isfinite(got).all(), f"{name} at dO x 2^{lg}"
+            _gate(r, got.float() / c, tol["atol"] * 2.0 ** -6, tol["rtol"], what=f"{name} at dO x 2^{lg}")
+    # beyond the bound: scale dO until the largest |dS| lies a factor 2 above 65504 / 2^p_shift
+    lg_over = int(np.ceil(np.log2(2 * 65504 / (ds_max * 2 ** shift))))
+    big = (base.float() * 2.0 ** lg_over).to(dtype)
+    if torch.isfinite(big).all():
+        _, _, g = _run(q.to(dtype), k.to(dtype), v.to(dtype), big, scale=scale)
+        finite = all(bool(torch.isfinite(t).all()) for t in g[:2])          # dQ and dK take dS
+        assert finite == (dtype == torch.bfloat16), "fp16 dS overflows past 65504 / 2^p_shift, bf16 does not"
+
+
 def test_bprop_closure_signature():
     B, N, S, D = 1, 2, 256, 128
     q, k, v, dO = (_gen((B, N, S, D), s).to(DEV) for s in (63, 64, 65, 66))
@@ -1318,6 +1357,28 @@ def _torch_cpu_causal_attention(q, k, v, dO, scale):
     return [torch.stack([o[i] for o in outs]).numpy() for i in range(len(outs[0]))]
 
 
+def _torch_cpu_attention(q, k, v, dO, scale, add_mask=None, drop=None, keep_prob=1.0):
+    """Every (batch, head) pair in torch fp32 on the host cores, with an additive mask [1|B,S,S] (-10000 where
+    masked) and a keep mask [B,N,S,S]: a second formulation (torch softmax, autograd for the gradients; the
+    row sum is taken before dropout, as the operator defines it).  The callers gate it against the fp64 oracle
+    on sampled heads before they use it for all heads."""
+    B, N, S, D = q.shape
+    outs = []
+    for b in range(B):
+        qf, kf, vf = (t[b].float().requires_grad_(True) for t in (q, k, v))
+        sc = torch.matmul(qf, kf.transpose(-1, -2)) * scale
+        if add_mask is not None:
+            sc = sc + add_mask[b if add_mask.shape[0] > 1 else 0]
+        P = torch.softmax(sc, -1)
+        L = torch.logsumexp(sc, -1)
+        if drop is not None:
+            P = P * (drop[b].float() / keep_prob)
+        O = torch.matmul(P, vf)
+        O.backward(dO[b].float())
+        outs.append((O.detach(), L.detach(), qf.grad, kf.grad, vf.grad))
+    return [torch.stack([o[i] for o in outs]).numpy() for i in range(5)]
+
+
 def test_full_size_fa2_causal_fwd_bwd():
     # B=4, N=16, S=2048, D=128, causal uint8 attn_mask, keep_prob = 1
     B, N, S, D = 4, 16, 2048, 128
@@ -1369,6 +1430,47 @@ def test_full_size_alibi():
         sl = (slice(b, b + 1), slice(h, h + 1))
         _check_all(q[sl], k[sl], v[sl], dO[sl], dict(scale=scale, attn_mask=tri, alibi=al[:, h:h + 1].float().numpy()),
                    (o[sl], lse[sl], tuple(t[sl] for t in g)))
+
+
+def test_full_size_alibi_full_bias_tensor():
+    # the same configuration with the bias as the full tensor alibi[h, i, j] = -slope_h (i - j), [1, N, S, S]
+    # (1 GiB in fp16): sampled heads against the oracle, every head against a second formulation
+    B, N, S, D = 2, 32, 4096, 128
+    q, k, v, dO = (_gen((B, N, S, D), 1011 + s).to(DEV) for s in range(4))
+    sl_ = torch.tensor(orc.alibi_slopes(N), dtype=torch.float32, device=DEV)
+    pos = torch.arange(S, dtype=torch.float32, device=DEV)
+    al_full = (-sl_[None, :, None, None] * (pos[None, None, :, None] - pos[None, None, None, :])).half()
+    scale = D ** -0.5
+    o, lse, g = _run(q, k, v, dO, scale=scale, mask_kind=_capi.MASK_CAUSAL, alibi=al_full, nxt=0)
+    tri = np.triu(np.ones((1, S, S), np.uint8), 1)
+    for b, h in _sample_heads(B, N, n=2, seed=5):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        bias = al_full[:, h:h + 1].float().cpu().numpy()       # the fp16 values the kernel reads
+        _check_all(q[sl].cpu(), k[sl].cpu(), v[sl].cpu(), dO[sl].cpu(), dict(scale=scale, attn_mask=tri, alibi=bias),
+                   (o[sl], lse[sl], tuple(t[sl] for t in g)))
+    # all 64 heads against a second formulation (torch fp32 on the device, one head at a time: additive -10000
+    # mask, torch softmax, autograd), which is held to the fp64 oracle on the sampled heads at a tenth of the gate
+    add = torch.triu(torch.full((S, S), -10000.0, device=DEV), 1)
+    sampled = set(_sample_heads(B, N, n=2, seed=5))
+    worst = 0.0
+    for b in range(B):
+        for h in range(N):
+            qf, kf, vf = (t[b, h].float().requires_grad_(True) for t in (q, k, v))
+            sc = qf @ kf.T * scale + al_full[0, h].float() + add
+            O = torch.softmax(sc, -1) @ vf
+            O.backward(dO[b, h].float())
+            got = (o[b, h], g[0][b, h], g[1][b, h], g[2][b, h])
+            for name, r, x in zip(("O", "dQ", "dK", "dV"), (O.detach(), qf.grad, kf.grad, vf.grad), got):
+                ok, ratio, _ = orc.tolerance_gate(r.cpu().numpy(), _np(x), atol=2.2e-3, rtol=1.1e-3)
+                worst = max(worst, ratio)
+                assert ok, f"{name} of head ({b}, {h}): {ratio:.3f}"
+            if (b, h) in sampled:
+                sl = (slice(b, b + 1), slice(h, h + 1))
+                okw = dict(scale=scale, attn_mask=tri, alibi=al_full[:, h:h + 1].float().cpu().numpy())
+                Oo, _ = orc.unfused_fwd(_np(q[sl]), _np(k[sl]), _np(v[sl]), **okw)
+                gr = orc.unfused_bwd(_np(q[sl]), _np(k[sl]), _np(v[sl]), _np(dO[sl]), **okw)
+                for r, t in zip((Oo,) + tuple(gr), (O.detach(), qf.grad, kf.grad, vf.grad)):
+                    assert orc.tolerance_gate(r[0, 0], t.cpu().numpy(), atol=2e-4, rtol=1e-4)[0]
 
 
 @pytest.mark.parametrize("dtype, D", [(torch.float16, 128), (torch.bfloat16, 64), (torch.float16, 80)])
@@ -1433,3 +1535,31 @@ def test_full_size_varlen_dropout():
     # padded keys receive exactly zero gradient
     for b in range(B):
         assert torch.count_nonzero(g[1][b, :, lens[b]:]) == 0 and torch.count_nonzero(g[2][b, :, lens[b]:]) == 0
+    # all 256 (batch, head) pairs (the XCD-grouped launch order with side inputs) against torch fp32 on the host,
+    # which is held to the fp64 oracle on the sampled heads at a tenth of the gate
+    add = torch.from_numpy(mask).float() * -10000.0
+    tO, tL, tdQ, tdK, tdV = _torch_cpu_attention(q, k, v, dO, scale, add_mask=add, drop=drop, keep_prob=0.9)
+    for b, h in _sample_heads(B, N, n=3, seed=3):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        okw = dict(scale=scale, attn_mask=mask[b:b + 1], drop_mask=drop[sl].numpy(), keep_prob=0.9)
+        O, L = orc.unfused_fwd(_np(q[sl]), _np(k[sl]), _np(v[sl]), **okw)
+        grads = orc.unfused_bwd(_np(q[sl]), _np(k[sl]), _np(v[sl]), _np(dO[sl]), **okw)
+        for ref, tt in zip((O,) + tuple(grads), (tO, tdQ, tdK, tdV)):
+            assert orc.tolerance_gate(ref, tt[sl], atol=2e-4, rtol=1e-4)[0]
+        assert np.max(np.abs(L - tL[sl])) < 1e-4
+    for name, ref, got in (("O", tO, o), ("dQ", tdQ, g[0]), ("dK", tdK, g[1]), ("dV", tdV, g[2])):
+        _gate(ref, got, 2.2e-3, 1.1e-3, what=name + " (all heads)")
+    assert np.max(np.abs(tL - _np(lse))) < 2e-4
+    # the same step with the keep mask drawn by the library and the mask's pre-pass results shared between the
+    # calls (the way the operator runs it): the zero-gradient property and the shapes of the masks hold there too
+    qd, kd, vd, dd = (t.to(DEV) for t in (q, k, v, dO))
+    p = _capi.make_params(qd, kd, vd, scale=scale, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_U8,
+                          attn_mask=torch.from_numpy(mask).to(DEV), drop_seed=99)
+    mb, db = _capi.attach_mask_bits(p, DEV), _capi.attach_drop_bits(p, DEV)
+    o2, lse2 = _capi.fa_fwd(p, qd)
+    p.mask_bits_filled = p.drop_bits_filled = 1
+    g2 = _capi.fa_bwd(p, qd, kd, vd, o2, dd, lse2)
+    assert mb is not None and db is not None
+    assert torch.allclose(lse2.cpu(), lse.cpu(), atol=1e-5)                      # LSE is taken before dropout
+    for b in range(B):
+        assert torch.count_nonzero(g2[1][b, :, lens[b]:]) == 0 and torch.count_nonzero(g2[2][b, :, lens[b]:]) == 0
