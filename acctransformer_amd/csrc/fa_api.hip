@@ -98,10 +98,9 @@ int validate(const acct_fa_params* p, bool backward) {
   if (p->D > 256) return fail(ACCT_E_HEADDIM, "head_dim too large, reduce head_dim and try again. (D=%d > 256)", p->D);
   if (p->D % 8 != 0) return fail(ACCT_E_HEADDIM, "head_dim %d is not a multiple of 8", p->D);
   (void)backward;
-  // bias and dropout variants are built for the head-dim classes 64, 80 and 128
-  const bool no_side = p->D == 40 || p->D > 128;
-  if (no_side && (p->alibi || p->drop_mask || (p->drop_philox && p->keep_prob < 1.f)))
-    return fail(ACCT_E_HEADDIM, "head_dim %d is built without the bias and dropout variants", p->D);
+  // bias variants are built for the head-dim classes 64, 80 and 128 (dropout: every head dim)
+  if ((p->D == 40 || p->D > 128) && p->alibi)
+    return fail(ACCT_E_HEADDIM, "head_dim %d is built without the bias variants", p->D);
   if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return fail(ACCT_E_PARAM, "scale must be positive and finite, got %g", (double)p->scale);
   if (!(p->keep_prob > 0.f && p->keep_prob <= 1.f)) return fail(ACCT_E_PARAM, "keep_prob must be in (0, 1], got %g", (double)p->keep_prob);
   if (p->prev_block_num < 0 || p->next_block_num < 0) return fail(ACCT_E_PARAM, "prev_block_num / next_block_num must be >= 0");

@@ -553,7 +553,7 @@ template <int D> constexpr int dkdv_groups() { return D > 128 ? 1 : 2; }
 // the hot variant must not carry that code's register pressure.
 template <typename T, int D, bool BIAS, bool DROP, bool MASKT, int NGK = 2>
 ACCT_DEV void fa_bwd_dkdv_body(const FaArgs& a) {
-  static_assert(NGK == 2 || (NGK == 1 && !BIAS && !DROP), "one key group per wave: the plain variants only");
+  static_assert(NGK == 2 || (NGK == 1 && !BIAS), "one key group per wave: no bias variants");
   using E = Elem<T>;
   using V8 = typename E::V8;
   using C = SwzCfg<D>;
@@ -1076,14 +1076,16 @@ static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
   return e;
 }
 
-// SIDE = false: head dims 40 and 160, built without the bias and dropout variants
-template <typename T, int D, bool SIDE = true>
+// SIDE: 2 = bias and dropout variants, 1 = the dropout variant only (head dims 40, 160, 256)
+template <typename T, int D, int SIDE = 2>
 static hipError_t launch_bwd_d(const FaArgs& a, int stages, hipStream_t st) {
   const bool bias = a.alibi != nullptr, drop = a.droprow != nullptr || a.dropcol != nullptr;
 #ifndef ACCT_DEV_BUILD
-  if constexpr (SIDE) {
-  if (bias) return drop ? launch_bwd_t<T, D, true, true>(a, stages, st) : launch_bwd_t<T, D, true, false>(a, stages, st);
-  if (drop) return launch_bwd_t<T, D, false, true>(a, stages, st);
+  if constexpr (SIDE == 2) {
+    if (bias) return drop ? launch_bwd_t<T, D, true, true>(a, stages, st) : launch_bwd_t<T, D, true, false>(a, stages, st);
+  }
+  if constexpr (SIDE >= 1) {
+    if (drop && !bias) return launch_bwd_t<T, D, false, true>(a, stages, st);
   }
 #endif
   if (bias || drop) return hipErrorNotSupported;       // (development build, head dims 40 / 160: plain variants only)
@@ -1107,16 +1109,16 @@ hipError_t launch_bwd(const FaArgs& a, int dtype, int Dr, int stages, hipStream_
     if (D == 128) return launch_bwd_d<f16, 128>(a, stages, st);
     if (D == 64) return launch_bwd_d<f16, 64>(a, stages, st);
     if (D == 80) return launch_bwd_d<f16, 80>(a, stages, st);
-    if (D == 40) return launch_bwd_d<f16, 40, false>(a, stages, st);
-    if (D == 160) return launch_bwd_d<f16, 160, false>(a, stages, st);
-    if (D == 256) return launch_bwd_d<f16, 256, false>(a, stages, st);
+    if (D == 40) return launch_bwd_d<f16, 40, 1>(a, stages, st);
+    if (D == 160) return launch_bwd_d<f16, 160, 1>(a, stages, st);
+    if (D == 256) return launch_bwd_d<f16, 256, 1>(a, stages, st);
   } else {
     if (D == 128) return launch_bwd_d<bf16, 128>(a, stages, st);
     if (D == 64) return launch_bwd_d<bf16, 64>(a, stages, st);
     if (D == 80) return launch_bwd_d<bf16, 80>(a, stages, st);
-    if (D == 40) return launch_bwd_d<bf16, 40, false>(a, stages, st);
-    if (D == 160) return launch_bwd_d<bf16, 160, false>(a, stages, st);
-    if (D == 256) return launch_bwd_d<bf16, 256, false>(a, stages, st);
+    if (D == 40) return launch_bwd_d<bf16, 40, 1>(a, stages, st);
+    if (D == 160) return launch_bwd_d<bf16, 160, 1>(a, stages, st);
+    if (D == 256) return launch_bwd_d<bf16, 256, 1>(a, stages, st);
   }
   return hipErrorInvalidValue;
 #endif

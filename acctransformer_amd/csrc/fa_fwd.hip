@@ -519,14 +519,16 @@ static hipError_t launch_fwd_t(const FaArgs& a, hipStream_t st) {
   }
 }
 
-// SIDE = false: the head dims of the inference operator, built without the bias and dropout variants
-template <typename T, int D, int QG, int NW, bool SIDE = true>
+// SIDE: 2 = bias and dropout variants, 1 = the dropout variant only (head dims 40, 160, 256)
+template <typename T, int D, int QG, int NW, int SIDE = 2>
 static hipError_t launch_fwd_q(const FaArgs& a, hipStream_t st) {
   const bool bias = a.alibi != nullptr, drop = a.droprow != nullptr || a.dropcol != nullptr;
 #ifndef ACCT_DEV_BUILD
-  if constexpr (SIDE) {
+  if constexpr (SIDE == 2) {
     if (bias) return drop ? launch_fwd_t<T, D, QG, NW, true, true>(a, st) : launch_fwd_t<T, D, QG, NW, true, false>(a, st);
-    if (drop) return launch_fwd_t<T, D, QG, NW, false, true>(a, st);
+  }
+  if constexpr (SIDE >= 1) {
+    if (drop && !bias) return launch_fwd_t<T, D, QG, NW, false, true>(a, st);
   }
 #endif
   if (bias || drop) return hipErrorNotSupported;       // (development build: plain variants only)
@@ -538,10 +540,10 @@ template <typename T, int D>
 static hipError_t launch_fwd_d(const FaArgs& a, int variant, hipStream_t st) {
   return variant == 3 ? launch_fwd_q<T, D, 1, 8>(a, st) : launch_fwd_q<T, D, 1, 4>(a, st);
 }
-// head dims 40 and 160: 32 rows per wave only
+// head dims 40 and 160: no bias variants
 template <typename T, int D>
 static hipError_t launch_fwd_plain(const FaArgs& a, int variant, hipStream_t st) {
-  return variant == 3 ? launch_fwd_q<T, D, 1, 8, false>(a, st) : launch_fwd_q<T, D, 1, 4, false>(a, st);
+  return variant == 3 ? launch_fwd_q<T, D, 1, 8, 1>(a, st) : launch_fwd_q<T, D, 1, 4, 1>(a, st);
 }
 
 #ifdef ACCT_DEV_BUILD
@@ -562,14 +564,14 @@ hipError_t launch_fwd(const FaArgs& a, int dtype, int Dr, int qg, hipStream_t st
     if (D == 80) return launch_fwd_d<f16, 80>(a, qg, st);
     if (D == 40) return launch_fwd_plain<f16, 40>(a, qg, st);
     if (D == 160) return launch_fwd_plain<f16, 160>(a, qg, st);
-    if (D == 256) return launch_fwd_q<f16, 256, 1, 4, false>(a, st);     // one wave per SIMD: 128 accumulator registers
+    if (D == 256) return launch_fwd_q<f16, 256, 1, 4, 1>(a, st);     // one wave per SIMD: 128 accumulator registers
   } else {
     if (D == 128) return launch_fwd_d<bf16, 128>(a, qg, st);
     if (D == 64) return launch_fwd_d<bf16, 64>(a, qg, st);
     if (D == 80) return launch_fwd_d<bf16, 80>(a, qg, st);
     if (D == 40) return launch_fwd_plain<bf16, 40>(a, qg, st);
     if (D == 160) return launch_fwd_plain<bf16, 160>(a, qg, st);
-    if (D == 256) return launch_fwd_q<bf16, 256, 1, 4, false>(a, st);
+    if (D == 256) return launch_fwd_q<bf16, 256, 1, 4, 1>(a, st);
   }
   return hipErrorInvalidValue;
 #endif

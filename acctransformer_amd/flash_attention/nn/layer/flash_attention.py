@@ -28,8 +28,9 @@ Differences from the reference Cell that a caller can see:
     new mask.  Pass `dropout_state=(seed, offset)` to `forward` to fix the
     stream of a call explicitly; the same pair reproduces the same mask.
   * Head dims: any multiple of 8 up to 256 (the reference admits multiples
-    of 16 up to 256); others raise when the op is called.  alibi_mask and
-    dropout need a head_dim of at most 128 other than 40.
+    of 16 up to 256); others raise in the constructor.  Dropout works at
+    every head dim; an alibi_mask needs a head_dim of at most 128 other
+    than 40 (the op raises otherwise).
 """
 from __future__ import annotations
 
@@ -68,6 +69,8 @@ class FlashAttention(torch.nn.Module):
         super().__init__()
         if head_dim > HEAD_DIM_MAX_LIMIT:
             raise ValueError("head_dim too large, reduce head_dim and try again.")
+        if head_dim <= 0 or head_dim % 8 != 0:
+            raise ValueError(f"head_dim must be a positive multiple of 8, but got {head_dim}")
         if alibi:
             raise ValueError("alibi not supported in the current version.")
         s = torch.tensor(1. / math.sqrt(math.sqrt(head_dim)), dtype=torch.float16)   # the reference's fp16 factor

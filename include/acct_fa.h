@@ -38,8 +38,8 @@ extern "C" {
 #define ACCT_E_SHAPE    (-2)   /* non-positive or inconsistent extent / stride */
 #define ACCT_E_DTYPE    (-3)   /* dtype is neither ACCT_F16 nor ACCT_BF16 */
 #define ACCT_E_HEADDIM  (-4)   /* D unsupported: not a multiple of 8, above 256 (L/flash_attention.py:26,105-106), or 40 / above 128 together
-                                  with a bias or dropout (kernels are built for 40, 64, 80, 128, 160, 256; other
-                                  multiples of 8 run on the next built size) */
+                                  with a bias (kernels are built for 40, 64, 80, 128, 160, 256; other multiples of 8 run
+                                  on the next built size; dropout is built for all of them) */
 #define ACCT_E_ARCH     (-5)   /* current device is not gfx950 */
 #define ACCT_E_LAUNCH   (-6)   /* HIP reported a launch error */
 #define ACCT_E_WORKSPACE (-7)  /* workspace missing or too small */
@@ -204,7 +204,7 @@ int acct_fa_bwd_static(const acct_fa_params* p, const void* O, const void* dO, c
  * (a 3-D input is also held to the reference's 1..64 rule for its last dimension, :104-112).  Writes q's
  * extents to y_dims (may be NULL) and returns ACCT_OK, else an error code; no device is touched.
  * The operator itself is acct_fa_fwd with scale = 1, mask_kind = NONE (head dims 40 and 160 are built
- * without the bias and dropout variants). */
+ * without the bias variants). */
 int acct_fa_infer_shape(const int64_t* q_dims, int q_rank, const int64_t* k_dims, int k_rank,
                         const int64_t* v_dims, int v_rank, int64_t* y_dims);
 

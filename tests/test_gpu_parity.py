@@ -718,9 +718,23 @@ def test_extra_head_dims_with_masks(D, dtype):
     tri = np.triu(np.ones((1, S, S), dtype=np.uint8), 1)
     _check_all(q, k, v, dO, dict(scale=D ** -0.5, attn_mask=tri),
                _run(q, k, v, dO, scale=D ** -0.5, mask_kind=_capi.MASK_CAUSAL, nxt=0), **tol)
-    # bias and dropout are not built for these head dims
+    # dropout at these head dims (the layer takes dropout_rate with any head dim up to 256,
+    # nn/layer/flash_attention.py:92-130,198-203): a byte mask with a padding mask on ragged lengths, and a
+    # keep mask drawn by the library from a seed pair under the causal mask
+    q, k, v, dO = (_gen(s, 830 + i, dtype) for i, s in enumerate([(B, N, Sq, D), (B, N, Sk, D), (B, N, Sk, D), (B, N, Sq, D)]))
+    drop = (rng.random((B, N, Sq, Sk)) < 0.8).astype(np.uint8)
+    pad = np.zeros((B, Sq, Sk), np.uint8); pad[0, :, 300:] = 1; pad[1, :, 411:] = 1
+    _check_all(q, k, v, dO, dict(scale=D ** -0.5, attn_mask=pad, drop_mask=drop, keep_prob=0.8),
+               _run(q, k, v, dO, scale=D ** -0.5, mask_kind=_capi.MASK_DENSE_U8, attn_mask=pad, drop_mask=drop, keep_prob=0.8), **tol)
+    q, k, v, dO = (_gen((B, N, S, D), 840 + i, dtype) for i in range(4))
+    v = (0.5 * v.float()).to(dtype)         # (first rows see one or two keys: see test_dense_mask_with_causal_diagonal_blocks)
+    keep = phx.dropout_keep_mask(B, N, S, S, 77, 5, 0.75)
+    _check_all(q, k, v, dO, dict(scale=D ** -0.5, attn_mask=tri, drop_mask=keep, keep_prob=phx.keep_threshold(0.75) / 256.0),
+               _run(q, k, v, dO, scale=D ** -0.5, mask_kind=_capi.MASK_CAUSAL, nxt=0, keep_prob=0.75, drop_seed=77, drop_offset=5), **tol)
+    # a bias is not built for these head dims
+    al = torch.zeros((1, 1, 1, S), dtype=dtype)
     with pytest.raises(_capi.AcctError) as e:
-        _run(q, k, v, dO, scale=1.0, keep_prob=0.9, drop_seed=3)
+        _run(q, k, v, dO, scale=1.0, alibi=al)
     assert e.value.code == -4
 
 
@@ -949,9 +963,11 @@ def test_random_configurations_on_the_eight_wave_kernels(block):
                 raise AssertionError(f"{c} head {(b, h)}: {e}") from e
 
 
-def test_layer_dropout_state_can_be_fixed_by_the_caller():
+@pytest.mark.parametrize("D", [64, 160])
+def test_layer_dropout_state_can_be_fixed_by_the_caller(D):
     # a forward that is run again (activation checkpointing) must draw the same mask: dropout_state fixes the stream
-    B, N, S, D = 1, 2, 256, 64
+    # (head dim 160: the layer takes dropout at every head dim it admits, nn/layer/flash_attention.py:92-130)
+    B, N, S = 1, 2, 256
     q, k, v = (_gen((B, N, S, D), s).to(DEV) for s in (860, 861, 862))
     layer = FlashAttention(head_dim=D, dropout_rate=0.2).train()
     a = layer(q, k, v, dropout_state=(99, 5))

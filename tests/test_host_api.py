@@ -153,7 +153,7 @@ def test_infer_shape_function():
     assert lib.acct_fa_infer_shape(None, 4, None, 4, None, 4, None) == -1
 
 
-def test_extra_head_dims_take_forward_and_backward_without_bias_and_dropout():
+def test_extra_head_dims_take_forward_and_backward_and_dropout_but_no_bias():
     lib = _capi.load()
     buf = (ctypes.c_char * 64)()
     a = ctypes.addressof(buf)
@@ -164,8 +164,14 @@ def test_extra_head_dims_take_forward_and_backward_without_bias_and_dropout():
         assert lib.acct_fa_fwd(ctypes.byref(p), None, None, None, 0, None) == -1
         # so does the backward (it gets past validation to the workspace check)
         assert lib.acct_fa_bwd(ctypes.byref(p), *([a] * 6), None, 0, None) == -7
+        # dropout is built for every head dim (the reference's layer takes dropout_rate with any head dim up to 256,
+        # nn/layer/flash_attention.py:92-130,198-203) ...
         p2 = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, keep_prob=0.9, drop_seed=1)
-        assert lib.acct_fa_fwd(ctypes.byref(p2), None, None, None, 0, None) == -4
+        assert lib.acct_fa_fwd(ctypes.byref(p2), None, None, None, 0, None) == -1
+        # ... a bias is not, and says so before anything is launched
+        p3 = _capi.make_params(q, q.clone(), q.clone(), scale=1.0, alibi=torch.zeros(1, 1, 1, 128, dtype=torch.float16))
+        assert lib.acct_fa_fwd(ctypes.byref(p3), None, None, None, 0, None) == -4
+        assert "bias" in lib.acct_last_error().decode()
 
 
 def test_no_cpu_fallback():
@@ -183,6 +189,9 @@ def test_layer_constructor_checks_match_reference():
         FlashAttention(head_dim=128, alibi=True)
     with pytest.raises(Exception, match="Strategy:foo not supported"):
         FlashAttention(head_dim=128, tiling_stgy_name="foo")
+    with pytest.raises(ValueError, match="multiple of 8"):
+        FlashAttention(head_dim=100)
+    FlashAttention(head_dim=160, dropout_rate=0.1)          # dropout at every head dim the layer admits
     layer = FlashAttention(head_dim=128, dropout_rate=0.1, prev_block_num=7, next_block_num=0)
     assert np.isclose(layer.scale, orc.flash_attention_layer_scale(128))
     assert layer.shard(((2, 4, 1, 1),) * 3) is layer and (layer.dp, layer.mp) == (2, 4)
