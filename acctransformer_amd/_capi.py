@@ -42,7 +42,7 @@ class AcctFaParams(ctypes.Structure):
         ("attn_mask", ctypes.c_void_p), ("drop_mask", ctypes.c_void_p), ("alibi", ctypes.c_void_p),
         ("drop_seed", ctypes.c_uint64), ("drop_offset", ctypes.c_uint32), ("drop_philox", ctypes.c_int32),
         ("drop_bits", ctypes.c_void_p), ("drop_bits_filled", ctypes.c_int32), ("drop_mask_kind", ctypes.c_int32),
-        ("mask_bits", ctypes.c_void_p), ("mask_bits_filled", ctypes.c_int32), ("reserved0", ctypes.c_int32),
+        ("mask_bits", ctypes.c_void_p), ("mask_bits_filled", ctypes.c_int32), ("grad_f32", ctypes.c_int32),
     ]
 
 
@@ -264,9 +264,10 @@ def fa_bwd(p, q, k, v, o, do, lse, workspace_bytes=None):
         tmp.copy_(do)
         do = tmp
     p.o_stride = _bhs_strides(o)
-    dq = torch.empty_strided(q.size(), q.stride(), dtype=q.dtype, device=q.device)
-    dk = torch.empty_strided(k.size(), k.stride(), dtype=k.dtype, device=k.device)
-    dv = torch.empty_strided(v.size(), v.stride(), dtype=v.dtype, device=v.device)
+    gdt = torch.float32 if p.grad_f32 else q.dtype       # (grad_f32: the reference's registered output type)
+    dq = torch.empty_strided(q.size(), q.stride(), dtype=gdt, device=q.device)
+    dk = torch.empty_strided(k.size(), k.stride(), dtype=gdt, device=k.device)
+    dv = torch.empty_strided(v.size(), v.stride(), dtype=gdt, device=v.device)
     nws = lib.acct_fa_bwd_workspace_bytes(ctypes.byref(p)) if workspace_bytes is None else int(workspace_bytes)
     ws = _workspace(nws, q.device)
     with torch.cuda.device(q.device):

@@ -69,6 +69,47 @@ int static_scratch(void** out) {
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// [B, N, S, D] rows of 2-byte floating-point elements -> float32, both sides with the same element strides
+// (grad_f32: the gradients in the reference's registered output type)
+template <typename T>
+__global__ void __launch_bounds__(256) cast_rows_to_f32_kernel(const T* src, float* dst, int N, int S, int D8, int64_t sb, int64_t sh,
+                                                              int64_t ss, long long chunks) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= chunks) return;
+  const int c = (int)(idx % D8);
+  const long long row = idx / D8;
+  const int s_ = (int)(row % S), h = (int)((row / S) % N);
+  const long long b = row / ((long long)S * N);
+  const int64_t off = b * sb + h * sh + (int64_t)s_ * ss + 8 * c;
+  typedef T t8 __attribute__((ext_vector_type(8)));
+  const t8 v = *reinterpret_cast<const t8*>(src + off);
+  acct::f32x4 lo = {(float)v[0], (float)v[1], (float)v[2], (float)v[3]}, hi = {(float)v[4], (float)v[5], (float)v[6], (float)v[7]};
+  *reinterpret_cast<acct::f32x4*>(dst + off) = lo;
+  *reinterpret_cast<acct::f32x4*>(dst + off + 4) = hi;
+}
+
+hipError_t cast_rows_to_f32(const void* src, float* dst, int dtype, int B, int N, int S, int D, int64_t sb, int64_t sh, int64_t ss, hipStream_t st) {
+  const long long chunks = (long long)B * N * S * (D / 8);
+  const unsigned grid = (unsigned)((chunks + 255) / 256);
+  if (dtype == ACCT_F16)
+    hipLaunchKernelGGL(cast_rows_to_f32_kernel<acct::f16>, dim3(grid), dim3(256), 0, st, (const acct::f16*)src, dst, N, S, D / 8, sb, sh, ss, chunks);
+  else
+    hipLaunchKernelGGL(cast_rows_to_f32_kernel<acct::bf16>, dim3(grid), dim3(256), 0, st, (const acct::bf16*)src, dst, N, S, D / 8, sb, sh, ss, chunks);
+  return hipGetLastError();
+}
+
+// elements between the first and one past the last element of a [B, N, S, D] tensor with these strides
+size_t span_elems(const int64_t st[3], int B, int N, int S, int D) {
+  if (st[0] == 0 && st[1] == 0 && st[2] == 0) return (size_t)B * N * S * D;
+  return (size_t)((B - 1) * st[0] + (N - 1) * st[1] + (S - 1) * st[2] + D);
+}
+// grad_f32: room for dQ, dK, dV in p->dtype, laid out like q, k, v
+size_t grad_tmp_bytes(const acct_fa_params* p, int which) {
+  if (!p->grad_f32) return 0;
+  const int64_t* st = which == 0 ? p->q_stride : (which == 1 ? p->k_stride : p->v_stride);
+  return align_up(span_elems(st, p->B, p->N, which == 0 ? p->Sq : p->Sk, p->D) * 2, 256);
+}
+
 bool strides_zero(const int64_t s[3]) { return s[0] == 0 && s[1] == 0 && s[2] == 0; }
 
 bool mask_is_dense(const acct_fa_params* p) { return p->mask_kind == ACCT_MASK_DENSE_U8 || p->mask_kind == ACCT_MASK_DENSE_F16; }
@@ -263,7 +304,7 @@ size_t acct_fa_drop_bits_bytes(const acct_fa_params* p) {
 // what the backward cannot do without: D and the exp2 offsets, the mask classes and bitmaps, the keep bits
 static size_t bwd_min_workspace_bytes(const acct_fa_params* p) {
   return 2 * align_up((size_t)p->B * p->N * p->Sq * sizeof(float), 256) + (p->mask_bits ? 0 : flag_bytes(p) + colbit_bytes(p)) +
-         (p->drop_bits ? 0 : droprow_bytes(p) + dropcol_bytes(p));
+         (p->drop_bits ? 0 : droprow_bytes(p) + dropcol_bytes(p)) + grad_tmp_bytes(p, 0) + grad_tmp_bytes(p, 1) + grad_tmp_bytes(p, 2);
 }
 
 size_t acct_fa_bwd_workspace_bytes(const acct_fa_params* p) {
@@ -365,6 +406,16 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
       if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "dropout bitmap kernel: %s", hipGetErrorString(e));
     }
   }
+  void* out_f32[3] = {dQ, dK, dV};
+  if (p->grad_f32) {
+    if (stages != (acct::kStageDq | acct::kStageDkDv)) return fail(ACCT_E_PARAM, "grad_f32 needs the fused acct_fa_bwd call");
+    if (((uintptr_t)dQ | (uintptr_t)dK | (uintptr_t)dV) & 15) return fail(ACCT_E_SHAPE, "dQ, dK and dV must be 16-byte aligned");
+    // the kernels write p->dtype tensors into the tail of the workspace; a conversion pass fills the caller's
+    char* tmp = (char*)workspace + need - grad_tmp_bytes(p, 0) - grad_tmp_bytes(p, 1) - grad_tmp_bytes(p, 2);
+    a.dq = tmp;
+    a.dk = tmp + grad_tmp_bytes(p, 0);
+    a.dv = tmp + grad_tmp_bytes(p, 0) + grad_tmp_bytes(p, 1);
+  }
   a.q_split = 1;
   if (want_dkdv) {
     const acct::DkdvSplit sp = acct::dkdv_split(p->B, p->N, p->Sq, p->Sk, p->D, n_cu);
@@ -376,6 +427,12 @@ static int bwd_impl(const acct_fa_params* p, const void* O, const void* dO, cons
   }
   hipError_t e = acct::launch_bwd(a, p->dtype, p->D, stages, st);
   if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "backward kernels: %s", hipGetErrorString(e));
+  if (p->grad_f32) {
+    e = cast_rows_to_f32(a.dq, (float*)out_f32[0], p->dtype, p->B, p->N, p->Sq, p->D, a.q_sb, a.q_sh, a.q_ss, st);
+    if (e == hipSuccess) e = cast_rows_to_f32(a.dk, (float*)out_f32[1], p->dtype, p->B, p->N, p->Sk, p->D, a.k_sb, a.k_sh, a.k_ss, st);
+    if (e == hipSuccess) e = cast_rows_to_f32(a.dv, (float*)out_f32[2], p->dtype, p->B, p->N, p->Sk, p->D, a.v_sb, a.v_sh, a.v_ss, st);
+    if (e != hipSuccess) return fail(ACCT_E_LAUNCH, "gradient conversion kernel: %s", hipGetErrorString(e));
+  }
   return ACCT_OK;
 }
 
@@ -389,6 +446,7 @@ int acct_fa_bwd_static(const acct_fa_params* p, const void* O, const void* dO, c
   g_err[0] = 0;
   int rc = validate(p, true);
   if (rc) return rc;
+  if (p->grad_f32) return fail(ACCT_E_PARAM, "acct_fa_bwd_static does not take grad_f32");
   const size_t need = bwd_min_workspace_bytes(p);
   if (need > (size_t)ACCT_FA_STATIC_SCRATCH_BYTES)
     return fail(ACCT_E_WORKSPACE, "acct_fa_bwd_static: this problem needs %zu bytes of scratch, the built-in buffer holds %zu; "

@@ -138,7 +138,13 @@ typedef struct acct_fa_params {
      step needs them once. */
   void*    mask_bits;
   int32_t  mask_bits_filled;
-  int32_t  reserved0;            /* must be 0 */
+  /* Backward only (field added in version 108): != 0 makes dQ, dK, dV float32 tensors (same element strides as
+     q, k, v), the output types the reference registers for its grad op before its bprop casts them to fp16
+     (T/flash_attention_impl.py:59-93,103-105,121-123) -- for graphs that keep that registration.  The values are
+     the p->dtype results converted (the kernels round once, from their fp32 accumulators, either way); the
+     workspace grows by room for the three p->dtype tensors (acct_fa_bwd_workspace_bytes accounts for it).
+     Not available through acct_fa_bwd_static, acct_fa_bwd_dq or acct_fa_bwd_dkdv. */
+  int32_t  grad_f32;
 } acct_fa_params;
 
 /* Forward: replaces the `flash_attention` TBE custom op, T/flash_attention_fwd.py:498-530

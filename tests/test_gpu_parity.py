@@ -1193,11 +1193,8 @@ def test_mindspore_aot_adapter_forward_and_backward():
     qd, kd, vd, dod = dev(q), dev(k), dev(v), dev(dO)
     mf, df = dev(torch.from_numpy(m8).half()), dev((torch.from_numpy(d8).float() / keep).half())
     o, lse = torch.empty_like(qd), torch.empty(B, N, S, dtype=torch.float32, device=DEV)
-    attrs = (ctypes.c_int32 * 2)(65536, 65536)
-
-    class Attrs(ctypes.Structure):
-        _fields_ = [("prev_block_num", ctypes.c_int32), ("next_block_num", ctypes.c_int32), ("scale", ctypes.c_float), ("keep_prob", ctypes.c_float)]
-    at = Attrs(65536, 65536, D ** -0.5, keep)
+    from test_host_api import MsAttrs
+    at = MsAttrs(MsAttrs.MAGIC, 65536, 65536, D ** -0.5, keep, 0)
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     sh, f16 = (B, N, S, D), "float16"
     plib = _capi.load()
@@ -1209,15 +1206,53 @@ def test_mindspore_aot_adapter_forward_and_backward():
     n, params, ndims, shapes, dtypes, _keep = ms_call_args(ops)
     assert lib.FlashAttentionFwd(n, params, ndims, shapes, dtypes, st, ctypes.addressof(at)) == 0, plib.acct_last_error().decode()
     dq, dk, dv = (torch.empty_like(t) for t in (qd, kd, vd))
-    # no workspace output declared: the adapter takes the entry point that needs none
-    ops = [(qd.data_ptr(), sh, f16), (kd.data_ptr(), sh, f16), (vd.data_ptr(), sh, f16), (o.data_ptr(), sh, f16),
+    gin = [(qd.data_ptr(), sh, f16), (kd.data_ptr(), sh, f16), (vd.data_ptr(), sh, f16), (o.data_ptr(), sh, f16),
            (dod.data_ptr(), sh, f16), (lse.data_ptr(), (B, N, S), "float32"), (mf.data_ptr(), (B, S, S), f16),
-           (df.data_ptr(), (B, N, S, S), f16), (None, (), f16),
-           (dq.data_ptr(), sh, f16), (dk.data_ptr(), sh, f16), (dv.data_ptr(), sh, f16)]
+           (df.data_ptr(), (B, N, S, S), f16), (None, (), f16)]
+    # no workspace output declared: refused, unless the attributes allow the built-in scratch (one buffer per GPU)
+    ops = gin + [(dq.data_ptr(), sh, f16), (dk.data_ptr(), sh, f16), (dv.data_ptr(), sh, f16)]
     n, params, ndims, shapes, dtypes, _keep = ms_call_args(ops)
+    assert lib.FlashAttentionGrad(n, params, ndims, shapes, dtypes, st, ctypes.addressof(at)) == -7
+    at.use_static_scratch = 1
     assert lib.FlashAttentionGrad(n, params, ndims, shapes, dtypes, st, ctypes.addressof(at)) == 0, plib.acct_last_error().decode()
     torch.cuda.synchronize()
     _check_all(q, k, v, dO, dict(scale=D ** -0.5, attn_mask=m8, drop_mask=d8, keep_prob=keep), (o, lse, (dq, dk, dv)))
+    # the reference's registration: float32 dq, dk, dv (flash_attention_impl.py:103-105), with a workspace output
+    # sized by the adapter's own query
+    at.use_static_scratch = 0
+    dq32, dk32, dv32 = (torch.empty(t.shape, dtype=torch.float32, device=DEV) for t in (qd, kd, vd))
+    lib.FlashAttentionGradWorkspaceBytes.restype = ctypes.c_size_t
+    lib.FlashAttentionGradWorkspaceBytes.argtypes = lib.FlashAttentionGrad.argtypes[:5] + [ctypes.c_void_p]
+    ops = gin + [(dq32.data_ptr(), sh, "float32"), (dk32.data_ptr(), sh, "float32"), (dv32.data_ptr(), sh, "float32")]
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(ops)
+    nws = lib.FlashAttentionGradWorkspaceBytes(n, params, ndims, shapes, dtypes, ctypes.addressof(at))
+    p.grad_f32 = 1
+    assert nws == plib.acct_fa_bwd_workspace_bytes(ctypes.byref(p)) and nws > 3 * qd.numel() * 2
+    ws2 = torch.empty(nws, dtype=torch.uint8, device=DEV)
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(ops + [(ws2.data_ptr(), (nws,), "uint8")])
+    assert lib.FlashAttentionGrad(n, params, ndims, shapes, dtypes, st, ctypes.addressof(at)) == 0, plib.acct_last_error().decode()
+    torch.cuda.synchronize()
+    for g16, g32 in ((dq, dq32), (dk, dk32), (dv, dv32)):
+        assert torch.equal(g16.float(), g32)               # the same values, in the wider type
+
+
+def test_float32_gradient_outputs_on_strided_inputs():
+    # grad_f32 through the C ABI on BSND views: float32 dQ, dK, dV with the element strides of q, k, v
+    B, N, S, D = 2, 3, 200, 64
+    base = [_gen((B, S, N, D), s).to(DEV) for s in (401, 402, 403, 404)]
+    q, k, v, dO = (t.permute(0, 2, 1, 3) for t in base)
+    p = _capi.make_params(q, k, v, scale=D ** -0.5, mask_kind=_capi.MASK_CAUSAL)
+    o, lse = _capi.fa_fwd(p, q)
+    ref = _capi.fa_bwd(p, q, k, v, o, dO, lse)
+    p.grad_f32 = 1
+    got = _capi.fa_bwd(p, q, k, v, o, dO, lse)
+    for a, b in zip(ref, got):
+        assert b.dtype == torch.float32 and b.stride() == a.stride() and torch.equal(a.float(), b)
+    lib = _capi.load()
+    buf = torch.empty(1 << 20, dtype=torch.uint8, device=DEV)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = lib.acct_fa_bwd_static(ctypes.byref(p), *([buf.data_ptr()] * 6), st)
+    assert rc == -8 and "grad_f32" in lib.acct_last_error().decode()
 
 
 # ---- the reference's CPU-sized configuration through the HIP path ------------------------------------

@@ -346,6 +346,13 @@ def _ms_lib():
     return lib
 
 
+class MsAttrs(ctypes.Structure):
+    """acct_ms_attrs of csrc/ms_aot_adapter.c"""
+    MAGIC = 0x41434354
+    _fields_ = [("magic", ctypes.c_uint32), ("prev_block_num", ctypes.c_int32), ("next_block_num", ctypes.c_int32),
+                ("scale", ctypes.c_float), ("keep_prob", ctypes.c_float), ("use_static_scratch", ctypes.c_int32)]
+
+
 def ms_call_args(operands):
     """(nparam, params, ndims, shapes, dtypes) of MindSpore's AOT convention from a list of (pointer or None, shape, dtype name)."""
     n = len(operands)
@@ -374,3 +381,36 @@ def test_mindspore_adapter_loads_and_validates_without_a_device():
     bad = list(good); bad[3] = (a, (1, 128, 128), "int32")
     n, params, ndims, shapes, dtypes, _keep = ms_call_args(bad)
     assert lib.FlashAttentionFwd(n, params, ndims, shapes, dtypes, None, None) == -3          # mask dtype
+    # output types: `output` in the operands' dtype, `rowsum` float32
+    bad = list(good); bad[7] = (a, sh[:3], "float16")
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(bad)
+    assert lib.FlashAttentionFwd(n, params, ndims, shapes, dtypes, None, None) == -3
+    # `extra` that is not an attribute block (MindSpore's own object, say) is refused, not read as attributes
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(good)
+    junk = (ctypes.c_char * 64)()
+    assert lib.FlashAttentionFwd(n, params, ndims, shapes, dtypes, None, ctypes.addressof(junk)) == -8
+    # a dropout mask without a keep probability below 1 (no attributes: keep_prob defaults to 1) is refused
+    bad = list(good); bad[4] = (a, (1, 2, 128, 128), "float16")
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(bad)
+    assert lib.FlashAttentionFwd(n, params, ndims, shapes, dtypes, None, None) == -8
+    # backward: dq, dk, dv all in the operands' dtype or all float32; a workspace output is required unless the
+    # attributes allow the shared built-in scratch
+    g = [(a, sh, "float16")] * 5 + [(a, sh[:3], "float32")] + [(None, (), "float16")] * 3 + [(a, sh, "float16")] * 3
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(g)
+    assert lib.FlashAttentionGrad(n, params, ndims, shapes, dtypes, None, None) == -7
+    mixed = list(g); mixed[10] = (a, sh, "float32")
+    n, params, ndims, shapes, dtypes, _keep = ms_call_args(mixed)
+    assert lib.FlashAttentionGrad(n, params, ndims, shapes, dtypes, None, None) == -3
+    # the accessor hook: the maintainer's init glue maps MindSpore's `extra` to the attribute block
+    at = MsAttrs(MsAttrs.MAGIC, 65536, 65536, 1.0, 1.0, 0)
+    ACC = ctypes.CFUNCTYPE(ctypes.c_void_p, ctypes.c_void_p)
+    acc = ACC(lambda extra: ctypes.addressof(at))
+    lib.acct_ms_set_attrs_accessor.argtypes = [ACC]
+    lib.acct_ms_set_attrs_accessor.restype = None
+    lib.acct_ms_set_attrs_accessor(acc)
+    try:
+        n, params, ndims, shapes, dtypes, _keep = ms_call_args(good)
+        rc = lib.FlashAttentionFwd(n, params, ndims, shapes, dtypes, None, ctypes.addressof(junk))
+        assert rc != -8                                    # the attributes were accepted (the call then needs a device)
+    finally:
+        lib.acct_ms_set_attrs_accessor(ctypes.cast(None, ACC))
