@@ -232,6 +232,11 @@ __global__ void __launch_bounds__(64) fa_drop_bits_kernel(const FaArgs a, uint32
   const int lane = threadIdx.x;
   const int kv = span * 1024 + 16 * lane;               // first of this lane's sixteen keys
   const bool vec = (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 15) == 0 && kv + 16 <= a.Sk;   // (16 elements: ES aligned 16-byte loads)
+  // Keys in a block that the attention mask's pre-pass classed 'skip' are never visited by the attention kernels:
+  // their keep bits are not read, so their mask bytes are not loaded either (this pass is bound by the bytes it
+  // reads; a padded batch skips a third to a half of them).
+  const bool dead = a.blkflags && kv < a.Sk &&
+                    a.blkflags[((int64_t)(a.mask_sb ? bh / a.N : 0) * a.Tr + qb) * a.Tc + kv / 128] == kBlkSkip;
   const int widx = 32 * span + (lane >> 1);             // this lane pair's word within the row
   const bool writer = rowbits && (lane & 1) == 0 && widx < a.droprow_w;
   uint32_t* rowout = rowbits + ((int64_t)bh * a.Sq + qb * 128 + 32 * i) * a.droprow_w + widx;
@@ -241,11 +246,11 @@ __global__ void __launch_bounds__(64) fa_drop_bits_kernel(const FaArgs a, uint32
   {
 #pragma unroll
     for (int e = 0; e < 16; e++) cw[e] = 0u;
-#pragma unroll 8
+#pragma unroll 16
     for (int r = 0; r < 32; r++) {
       const int rr = 32 * i + r;
       uint32_t nz = 0;                                  // bit e: this lane's key e of the row is kept
-      if (rr < nrow) {
+      if (rr < nrow && !dead) {
         if (vec) {
 #pragma unroll
           for (int h = 0; h < ES; h++) {

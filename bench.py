@@ -64,6 +64,171 @@ def cpu_baseline(budget_s=12.0):
     }
 
 
+class PowerSampler:
+    """Board power from the amdgpu hwmon files in sysfs (power1_input, microwatts; power1_cap = the limit the
+    power management holds the board to), read every 20 ms by a host thread while the GPU works."""
+
+    def __init__(self):
+        import glob
+        self.dir = next(iter(sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*"))), None)
+        self.samples, self._stop, self._thread = [], False, None
+
+    def _read(self, name):
+        try:
+            with open(os.path.join(self.dir, name)) as f:
+                return int(f.read())
+        except Exception:
+            return None
+
+    def start(self):
+        import threading
+        if self.dir is None or self._read("power1_input") is None:
+            return False
+        self.samples, self._stop = [], False
+
+        def loop():
+            while not self._stop:
+                v = self._read("power1_input")
+                if v is not None:
+                    self.samples.append(v / 1e6)
+                time.sleep(0.02)
+        self._thread = threading.Thread(target=loop, daemon=True)
+        self._thread.start()
+        return True
+
+    def stop(self):
+        if self._thread is None:
+            return None
+        self._stop = True
+        self._thread.join()
+        self._thread = None
+        s = self.samples[len(self.samples) // 3:]           # (the first third: the reading still rises)
+        if not s:
+            return None
+        cap = self._read("power1_cap")
+        return {"source": os.path.join(self.dir, "power1_input"), "samples": len(s), "mean_w": round(sum(s) / len(s), 1),
+                "max_w": round(max(s), 1), "cap_w": None if cap is None else cap / 1e6}
+
+
+def run_other_configs(args, lib, dev, st, stream, g, D, scale, check, only):
+    """The configurations of the benchmark line besides the timed one.  `only`: run just the one of that name
+    (for a profiler run over a single configuration) with `args.steps` steps."""
+    import ctypes
+    import torch
+    from acctransformer_amd import _capi
+    P = ctypes.byref
+    other = {}
+
+    def run_config(name, pp, qq, kk, vv, dd, flops, side_bytes, n=10):
+        oo, ll = torch.empty_like(qq), torch.empty(qq.shape[:3], dtype=torch.float32, device=dev)
+        g3 = [torch.empty_like(t) for t in (qq, kk, vv)]
+        pp.o_stride = _capi._bhs_strides(oo)
+        # with dropout, the forward call packs (or draws) the keep bits into a buffer that the backward call of
+        # the same step reads (drop_bits / drop_bits_filled of the C ABI), as the Python operator does; the same
+        # for what the pre-pass derives from a mask tensor (mask_bits): once per step, in the forward call
+        bits = _capi.attach_drop_bits(pp, dev)
+        mbits = _capi.attach_mask_bits(pp, dev)
+        nw = max(lib.acct_fa_bwd_workspace_bytes(P(pp)), lib.acct_fa_fwd_workspace_bytes(P(pp)), 256)
+        w = torch.empty(nw, dtype=torch.uint8, device=dev)
+
+        def one():
+            pp.drop_bits_filled = 0
+            pp.mask_bits_filled = 0
+            check(lib.acct_fa_fwd(P(pp), oo.data_ptr(), ll.data_ptr(), w.data_ptr(), nw, st))
+            pp.drop_bits_filled = 1 if bits is not None else 0
+            pp.mask_bits_filled = 1 if mbits is not None else 0
+            check(lib.acct_fa_bwd(P(pp), oo.data_ptr(), dd.data_ptr(), ll.data_ptr(), g3[0].data_ptr(), g3[1].data_ptr(),
+                                  g3[2].data_ptr(), w.data_ptr(), nw, st))
+        # untimed: the inputs were drawn on the host while the GPU sat idle, and the clock needs a few tenths
+        # of a second under load to settle again
+        t_end = time.perf_counter() + max(args.settle_seconds, 0.0) / 2
+        while True:
+            for _ in range(3):
+                one()
+            torch.cuda.synchronize()
+            if time.perf_counter() >= t_end:
+                break
+        if only is not None:
+            n = args.steps
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(n):
+            one()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / n
+        io = 8 * qq.numel() * qq.element_size() + 2 * ll.numel() * 4 + side_bytes
+        other[name] = {"ms_per_step": round(ms, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
+                       "algorithmic_hbm_gb_per_step": round(io / 1e9, 3), "achieved_hbm_gbps": round(io / (ms * 1e-3) / 1e9, 1),
+                       "hbm_peak_gbps": 8000.0}
+
+    want = lambda name: only is None or only == name
+    # ALiBi + causal, B2 N32 S4096 D128: bias -slope_h (i - j), as a full [1,N,S,S] tensor and in the
+    # reference's row-bias form [1,N,1,S] (slope_h j: the row constant cancels in the softmax)
+    names3 = ("alibi_causal_B2_N32_S4096_row_bias", "alibi_causal_B2_N32_S4096_full_bias")
+    if any(want(nm) for nm in names3):
+        B3, N3, S3 = 2, 32, 4096
+        q3, k3, v3, d3 = (torch.randn(B3, N3, S3, D, generator=g).half().to(dev) for _ in range(4))
+        slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / N3) for h in range(N3)], device=dev)
+        pos = torch.arange(S3, device=dev, dtype=torch.float32)
+        fl3 = 14.0 * B3 * N3 * S3 * S3 * D * 0.5
+        for nm in names3:
+            if not want(nm):
+                continue
+            if nm.endswith("row_bias"):
+                al = (slopes[None, :, None, None] * pos[None, None, None, :]).half()
+            else:
+                al = (-slopes[None, :, None, None] * (pos[None, None, :, None] - pos[None, None, None, :])).half()
+            pp = _capi.make_params(q3, k3, v3, scale=scale, next_block_num=0, mask_kind=_capi.MASK_CAUSAL, alibi=al)
+            run_config(nm, pp, q3, k3, v3, d3, fl3, 2 * al.numel() * 2)      # the bias is read by the forward and by the backward
+            del al
+        del q3, k3, v3, d3
+    # padded batch + dropout, B16 N16 S1024 D128: key-padding mask [B,S,S] uint8, lengths U[256,1024]; dropout
+    # mask uint8 [B,N,S,S] Bernoulli(0.9)
+    names5 = ("padded_dropout_B16_N16_S1024_mask_tensor", "padded_dropout_B16_N16_S1024_fp16_mask_tensors",
+              "padded_dropout_B16_N16_S1024_seed_pair")
+    if any(want(nm) for nm in names5):
+        B5, N5, S5 = 16, 16, 1024
+        g5 = torch.Generator(device="cpu").manual_seed(1005)
+        q5, k5, v5, d5 = (torch.randn(B5, N5, S5, D, generator=g5).half().to(dev) for _ in range(4))
+        # (a generator of its own for the lengths: a draw whose mean, 0.4986 S, is that of the draw the earlier
+        # runs of this benchmark happened to take from the shared stream, so that the figures stay comparable)
+        lens = torch.randint(256, S5 + 1, (B5,), generator=torch.Generator(device="cpu").manual_seed(1898))
+        m5 = (torch.arange(S5)[None, None, :] >= lens[:, None, None]).expand(B5, S5, S5).to(torch.uint8).contiguous().to(dev)
+        dr5 = (torch.rand(B5, N5, S5, S5, generator=g5) < 0.9).to(torch.uint8).to(dev)
+        f5 = float(lens.float().mean()) / S5
+        fl5 = 14.0 * B5 * N5 * S5 * S5 * D * f5
+        if want(names5[0]):
+            pp = _capi.make_params(q5, k5, v5, scale=scale, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m5, drop_mask=dr5)
+            run_config(names5[0], pp, q5, k5, v5, d5, fl5, 2 * (m5.numel() + dr5.numel()))
+        if want(names5[1]):
+            # the same masks in the reference's own form: fp16 attn_mask (1 = masked) and fp16 {0, 1/keep_prob} dropout mask
+            m5f, dr5f = m5.half(), (dr5.half() / 0.9).half()
+            pp = _capi.make_params(q5, k5, v5, scale=scale, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_F16, attn_mask=m5f, drop_mask=dr5f)
+            run_config(names5[1], pp, q5, k5, v5, d5, fl5, 2 * 2 * (m5.numel() + dr5.numel()))
+            del m5f, dr5f
+        if want(names5[2]):
+            pp = _capi.make_params(q5, k5, v5, scale=scale, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m5, drop_seed=1234)
+            run_config(names5[2], pp, q5, k5, v5, d5, fl5, 2 * m5.numel())
+        other["padded_dropout_unmasked_fraction"] = round(f5, 4)
+        del q5, k5, v5, d5, m5, dr5
+    # the reference's own performance test (tests/train/flash_attention/st/test_fa_perf.py:16-58): the raw op on
+    # (4, 8, 4096, 128) with uniform [0, 1) inputs, a (1, S, S) fp16 causal attn_mask and an fp16 {0, 1/keep_prob}
+    # dropout mask of rate 0.1, forward and grad
+    nm = "reference_perf_test_B4_N8_S4096_fp16_masks_dropout"
+    if want(nm):
+        B6, N6, S6 = 4, 8, 4096
+        g6 = torch.Generator(device="cpu").manual_seed(1006)
+        q6, k6, v6 = (torch.rand(B6, N6, S6, D, generator=g6).half().to(dev) for _ in range(3))
+        d6 = torch.randn(B6, N6, S6, D, generator=g6).half().to(dev)
+        m6 = torch.triu(torch.ones(1, S6, S6, dtype=torch.float16, device=dev), 1)
+        dr6 = ((torch.rand(B6, N6, S6, S6, device=dev) < 0.9).half() / 0.9).half()
+        pp = _capi.make_params(q6, k6, v6, scale=1.0, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_F16, attn_mask=m6, drop_mask=dr6)
+        run_config(nm, pp, q6, k6, v6, d6, 14.0 * B6 * N6 * S6 * S6 * D * 0.5, 2 * 2 * (m6.numel() + dr6.numel()), n=5)
+        del q6, k6, v6, d6, m6, dr6
+    return other
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -76,6 +241,12 @@ def main():
                     help="skip the register-only MFMA rate measurement (the `mfma_sustained` key of the JSON line)")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the ALiBi and padded-batch + dropout configurations (extra keys of the JSON line)")
+    ap.add_argument("--data", choices=("randn", "const", "zeros"), default="randn",
+                    help="q, k, v, dO of the timed workload: N(0,1) (the benchmark's), one value in every element, or "
+                         "zeros -- the same instructions on operands that toggle less and draw less power")
+    ap.add_argument("--only-config", default=None,
+                    help="run one of the `other_configs` by name for --steps steps and print its entry only (so that a "
+                         "profile covers that configuration alone)")
     ap.add_argument("--no-dense-pass", action="store_true",
                     help="skip the untimed dense-mask and TriangleAttention comparison passes (so that a profile covers the timed workload only)")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
@@ -101,7 +272,19 @@ def main():
 
     B, N, S, D = 4, 16, 2048, 128
     g = torch.Generator(device="cpu").manual_seed(1001)
+    if args.only_config:
+        stream = torch.cuda.current_stream()
+        st = ctypes.c_void_p(stream.cuda_stream)
+
+        def check(rc):
+            if rc != 0:
+                raise RuntimeError(lib.acct_last_error().decode())
+        print(json.dumps(run_other_configs(args, lib, dev, st, stream, g, D, D ** -0.5, check, args.only_config)))
+        return
     q, k, v, dO = (torch.randn(B, N, S, D, generator=g).half().to(dev) for _ in range(4))
+    if args.data != "randn":
+        for t in (q, k, v, dO):
+            t.fill_(0.25 if args.data == "const" else 0.0)
     attn_mask = torch.triu(torch.ones(1, S, S, dtype=torch.uint8, device=dev), 1)
     scale = D ** -0.5
     # The timed workload: the uint8 attn_mask tensor is read by the library.  Its pre-pass classifies the 128x128
@@ -148,6 +331,8 @@ def main():
     # Clock settle: the first ~100 steps after an idle period run on clocks that are still moving (measured:
     # up to 16 % slower), whatever --warmup says.  Keep stepping untimed until half a second of work has gone
     # through the GPU; the timed region below then starts on settled clocks.
+    power = PowerSampler()
+    power.start()                                         # sampled over the settle phase and the timed region
     t_s = time.perf_counter()
     settle_steps = 0
     while time.perf_counter() - t_s < args.settle_seconds:
@@ -177,6 +362,7 @@ def main():
         if e: e[3].record(stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    board_power = power.stop()
     ms_step = wall * 1e3 / K
     t_fwd = sum(e[0].elapsed_time(e[1]) for e in ev.values()) / len(ev)
     t_dq = sum(e[1].elapsed_time(e[2]) for e in ev.values()) / len(ev)
@@ -226,85 +412,13 @@ def main():
                "block_skip_speedup": round(ms_all / ms_tri, 3)}
         del qt, kt, vt, mt
 
-    # The other two training configurations (untimed for `value`; extra keys of the line): forward + fused
+    # The other training configurations (untimed for `value`; extra keys of the line): forward + fused
     # backward through the C ABI, kernel time by HIP events on the launch stream, algorithmic flops by the same
     # convention, and the algorithmic HBM bytes per step (every operand read or written once: q, k, v, O, dO,
     # dQ, dK, dV, LSE twice, and the side inputs once per call that reads them) over the same time.
     other = None
     if not args.no_other_configs:
-        other = {}
-
-        def run_config(name, pp, qq, kk, vv, dd, flops, side_bytes, n=10):
-            oo, ll = torch.empty_like(qq), torch.empty(qq.shape[:3], dtype=torch.float32, device=dev)
-            g3 = [torch.empty_like(t) for t in (qq, kk, vv)]
-            pp.o_stride = _capi._bhs_strides(oo)
-            # with dropout, the forward call packs (or draws) the keep bits into a buffer that the backward call of
-            # the same step reads (drop_bits / drop_bits_filled of the C ABI), as the Python operator does
-            bits = _capi.attach_drop_bits(pp, dev)
-            nw = max(lib.acct_fa_bwd_workspace_bytes(P(pp)), lib.acct_fa_fwd_workspace_bytes(P(pp)), 256)
-            w = torch.empty(nw, dtype=torch.uint8, device=dev)
-
-            def one():
-                pp.drop_bits_filled = 0
-                check(lib.acct_fa_fwd(P(pp), oo.data_ptr(), ll.data_ptr(), w.data_ptr(), nw, st))
-                pp.drop_bits_filled = 1 if bits is not None else 0
-                check(lib.acct_fa_bwd(P(pp), oo.data_ptr(), dd.data_ptr(), ll.data_ptr(), g3[0].data_ptr(), g3[1].data_ptr(),
-                                      g3[2].data_ptr(), w.data_ptr(), nw, st))
-            # untimed: the inputs were drawn on the host while the GPU sat idle, and the clock needs a few tenths
-            # of a second under load to settle again
-            t_end = time.perf_counter() + max(args.settle_seconds, 0.0) / 2
-            while True:
-                for _ in range(3):
-                    one()
-                torch.cuda.synchronize()
-                if time.perf_counter() >= t_end:
-                    break
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for _ in range(n):
-                one()
-            e1.record(stream)
-            torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1) / n
-            io = 8 * qq.numel() * qq.element_size() + 2 * ll.numel() * 4 + side_bytes
-            other[name] = {"ms_per_step": round(ms, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
-                           "algorithmic_hbm_gb_per_step": round(io / 1e9, 3), "achieved_hbm_gbps": round(io / (ms * 1e-3) / 1e9, 1),
-                           "hbm_peak_gbps": 8000.0}
-
-        # ALiBi + causal, B2 N32 S4096 D128: bias -slope_h (i - j), as a full [1,N,S,S] tensor and in the
-        # reference's row-bias form [1,N,1,S] (slope_h j: the row constant cancels in the softmax)
-        B3, N3, S3 = 2, 32, 4096
-        q3, k3, v3, d3 = (torch.randn(B3, N3, S3, D, generator=g).half().to(dev) for _ in range(4))
-        slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / N3) for h in range(N3)], device=dev)
-        pos = torch.arange(S3, device=dev, dtype=torch.float32)
-        al_row = (slopes[None, :, None, None] * pos[None, None, None, :]).half()
-        al_full = (-slopes[None, :, None, None] * (pos[None, None, :, None] - pos[None, None, None, :])).half()
-        fl3 = 14.0 * B3 * N3 * S3 * S3 * D * 0.5
-        for nm, al in (("alibi_causal_B2_N32_S4096_row_bias", al_row), ("alibi_causal_B2_N32_S4096_full_bias", al_full)):
-            pp = _capi.make_params(q3, k3, v3, scale=scale, next_block_num=0, mask_kind=_capi.MASK_CAUSAL, alibi=al)
-            run_config(nm, pp, q3, k3, v3, d3, fl3, 2 * al.numel() * 2)      # the bias is read by the forward and by the backward
-        del q3, k3, v3, d3, al_row, al_full
-        # padded batch + dropout, B16 N16 S1024 D128: key-padding mask [B,S,S] uint8, lengths U[256,1024]; dropout
-        # mask uint8 [B,N,S,S] Bernoulli(0.9)
-        B5, N5, S5 = 16, 16, 1024
-        q5, k5, v5, d5 = (torch.randn(B5, N5, S5, D, generator=g).half().to(dev) for _ in range(4))
-        lens = torch.randint(256, S5 + 1, (B5,), generator=g)
-        m5 = (torch.arange(S5)[None, None, :] >= lens[:, None, None]).expand(B5, S5, S5).to(torch.uint8).contiguous().to(dev)
-        dr5 = (torch.rand(B5, N5, S5, S5, generator=g) < 0.9).to(torch.uint8).to(dev)
-        f5 = float(lens.float().mean()) / S5
-        fl5 = 14.0 * B5 * N5 * S5 * S5 * D * f5
-        pp = _capi.make_params(q5, k5, v5, scale=scale, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m5, drop_mask=dr5)
-        run_config("padded_dropout_B16_N16_S1024_mask_tensor", pp, q5, k5, v5, d5, fl5, 2 * (m5.numel() + dr5.numel()))
-        # the same masks in the reference's own form: fp16 attn_mask (1 = masked) and fp16 {0, 1/keep_prob} dropout mask
-        m5f, dr5f = m5.half(), (dr5.half() / 0.9).half()
-        pp = _capi.make_params(q5, k5, v5, scale=scale, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_F16, attn_mask=m5f, drop_mask=dr5f)
-        run_config("padded_dropout_B16_N16_S1024_fp16_mask_tensors", pp, q5, k5, v5, d5, fl5, 2 * 2 * (m5.numel() + dr5.numel()))
-        del m5f, dr5f
-        pp = _capi.make_params(q5, k5, v5, scale=scale, keep_prob=0.9, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m5, drop_seed=1234)
-        run_config("padded_dropout_B16_N16_S1024_seed_pair", pp, q5, k5, v5, d5, fl5, 2 * m5.numel())
-        other["padded_dropout_unmasked_fraction"] = round(f5, 4)
-        del q5, k5, v5, d5, m5, dr5
-
+        other = run_other_configs(args, lib, dev, st, stream, g, D, scale, check, None)
     if args.calib_copy_mib > 0:
         src = torch.ones(args.calib_copy_mib * (1 << 18), dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
@@ -338,14 +452,21 @@ def main():
     # operands toggle (the clock follows the power drawn); the benchmark's N(0,1) data is the varying case.
     mfma = None
     if not args.no_mfma_probe:
-        rates, clocks = {}, {}
+        rates, clocks, watts = {}, {}, {}
         for key, varying in (("varying_operands", 1), ("constant_operands", 0)):
             r, ghz = ctypes.c_double(0.0), ctypes.c_double(0.0)
-            check(lib.acct_probe_mfma_clock(varying, ctypes.byref(r), ctypes.byref(ghz), st))
+            power.start()
+            t_p = time.perf_counter()
+            while True:                                   # (repeated for half a second so that the power reading settles)
+                check(lib.acct_probe_mfma_clock(varying, ctypes.byref(r), ctypes.byref(ghz), st))
+                if time.perf_counter() - t_p > 0.5:
+                    break
+            w = power.stop()
             rates[key] = round(r.value, 1)
             clocks[key] = round(ghz.value, 3)
+            watts[key] = None if w is None else w["mean_w"]
         # (shader clock a wave saw inside the loop: an MFMA takes 32 clocks either way, the power drawn sets the clock)
-        mfma = {"unit": "TFLOP/s", "instruction": "v_mfma_f32_32x32x16_f16", **rates, "shader_clock_ghz": clocks,
+        mfma = {"unit": "TFLOP/s", "instruction": "v_mfma_f32_32x32x16_f16", **rates, "shader_clock_ghz": clocks, "board_power_w": watts,
                 "frac_of_nominal_peak": round(rates["varying_operands"] / PEAK_FP16_TFLOPS, 4),
                 "dominant_kernel_frac_of_sustained": round(achieved / rates["varying_operands"], 4)}
     out = {
@@ -363,6 +484,8 @@ def main():
         "triangle_block_skip": tri,
         "other_configs": other,
         "clock_settle": {"seconds": round(settle_s, 3), "steps": settle_steps},
+        "board_power": board_power,
+        "input_data": args.data,
         "mfma_sustained": mfma,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": traffic_bytes[dom]},

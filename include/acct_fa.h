@@ -121,7 +121,9 @@ typedef struct acct_fa_params {
      caller keeps from the forward to the backward call, a call with drop_bits_filled == 0 runs the pre-pass
      into that buffer and a call with drop_bits_filled != 0 reads what an earlier call left there.  The
      caller sets drop_bits_filled after the first call returns; the bits depend on drop_mask or on
-     (drop_seed, drop_offset, keep_prob) and on B, N, Sq, Sk only. */
+     (drop_seed, drop_offset, keep_prob) and on B, N, Sq, Sk; with a dense attn_mask the bits of the 128x128
+     blocks that the mask hides completely are left out (no kernel reads them), so the buffer belongs to the
+     calls of one step on one attn_mask. */
   void*    drop_bits;
   int32_t  drop_bits_filled;
   int32_t  drop_mask_kind;       /* ACCT_DROP_* (field added in version 104; 0 = the uint8 form) */
