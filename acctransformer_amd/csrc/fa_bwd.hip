@@ -18,6 +18,8 @@
 #include "fa_common.hpp"
 #include "fa_launch.hpp"
 
+#include <type_traits>
+
 namespace acct {
 template <typename T>
 ACCT_DEV typename Elem<T>::V8 pack8(const float* x) {
@@ -1034,7 +1036,16 @@ __global__ void __launch_bounds__(512) fa_bwd_dkdv_kernel(const FaArgs a) {
 template <typename T, int D, bool BIAS, bool DROP>
 static hipError_t launch_bwd_t(FaArgs a, int stages, hipStream_t st) {
   hipError_t e = hipSuccess;
-  if (stages & kStageDq) {
+  bool dq_done = false;
+  if constexpr (D == 128 && !BIAS && !DROP) {
+    // head dim 128 without side inputs on aligned lengths: the kernel with 64 query rows per wave
+    if ((stages & kStageDq) && dq64_applicable(a)) {
+      e = launch_bwd_dq64(a, std::is_same<T, bf16>::value ? 1 : 0, st);
+      if (e != hipSuccess) return e;
+      dq_done = true;
+    }
+  }
+  if ((stages & kStageDq) && !dq_done) {
     constexpr int QG = 1, NW = D > 128 ? 4 : 8;          // (wide head dims: one wave per SIMD has the registers)
     constexpr int BM = 32 * QG * NW;
     using CS = SwzCfg<D>;

@@ -30,6 +30,10 @@ hipError_t launch_fwd(const FaArgs& a, int dtype, int D, int qg, hipStream_t st)
 enum : int { kStageDq = 1, kStageDkDv = 2 };
 hipError_t launch_bwd(const FaArgs& a, int dtype, int D, int stages, hipStream_t st);
 
+// the dQ kernel with 64 query rows per wave (fa_bwd_dq64.hip): head dim 128, no side inputs, aligned lengths
+bool dq64_applicable(const FaArgs& a);
+hipError_t launch_bwd_dq64(FaArgs a, int dtype, hipStream_t st);
+
 // false when the kernel translation units were compiled with a reduced variant set (ACCT_DEV_BUILD)
 bool launch_variants_complete();
 

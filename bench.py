@@ -252,6 +252,12 @@ def main():
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also run an elementwise fp32 copy kernel over this many MiB (5 launches) after the timed "
                          "region: a known-size reference for scaling profiler byte counters")
+    ap.add_argument("--lib", default=None,
+                    help="load this build of libacct_fa.so instead of the in-tree one (a timing build made by "
+                         "`make -C acctransformer_amd/csrc leave-out LEAVE_OUT=...`)")
+    ap.add_argument("--kernel-times", action="store_true",
+                    help="print the time of each of the three kernels alone (HIP events over --steps launches) on the "
+                         "benchmark shape, with the mask declared as none and as causal, and exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the single-GPU attention hot path: run it with --gpus 1 "
@@ -268,6 +274,8 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.lib:
+        _capi._LIB_PATH = os.path.abspath(args.lib)
     lib = _capi.load()
 
     B, N, S, D = 4, 16, 2048, 128
@@ -324,6 +332,30 @@ def main():
         fwd(pp)
         pp.mask_bits_filled = 1 if pp.mask_bits else 0
         bwd_dq(pp); bwd_dkdv(pp)
+
+    if args.kernel_times:
+        out = {"lib": _capi.lib_path(), "data": args.data, "launches": args.steps, "unit": "us", "kernels": {}}
+        for name, kind in (("mask_none", _capi.MASK_NONE), ("mask_causal", _capi.MASK_CAUSAL)):
+            pk = _capi.make_params(q, k, v, scale=scale, mask_kind=kind)
+            pk.o_stride = _capi._bhs_strides(o)
+            fwd(pk)
+            row = {}
+            for kname, fn in (("fa_fwd", fwd), ("fa_bwd_dq", bwd_dq), ("fa_bwd_dkdv", bwd_dkdv)):
+                t_s = time.perf_counter()
+                while time.perf_counter() - t_s < args.settle_seconds:
+                    for _ in range(20):
+                        fn(pk)
+                    torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(args.steps):
+                    fn(pk)
+                e1.record(stream)
+                torch.cuda.synchronize()
+                row[kname] = round(e0.elapsed_time(e1) * 1e3 / args.steps, 2)
+            out["kernels"][name] = row
+        print(json.dumps(out))
+        return
 
     for _ in range(args.warmup):
         step(p_dense)

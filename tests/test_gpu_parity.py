@@ -358,6 +358,36 @@ def test_block_band(prev, nxt):
     _check_all(q, k, v, dO, okw, _run(q, k, v, dO, scale=D ** -0.5, prev=prev, nxt=nxt))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Sq, Sk, causal", [(256, 64, False), (256, 192, False), (512, 512, True), (768, 320, True),
+                                            (512, 1024, True), (256, 64, True), (1024, 2048, False)])
+def test_dq_kernel_with_64_rows_per_wave(dtype, Sq, Sk, causal):
+    # shapes the hand-scheduled dQ kernel takes (head dim 128, 256-row query blocks, 64-key tiles, no side
+    # inputs): one tile, an odd tile count, diagonals that end inside and past the keys, rows past the last key
+    B, N, D = 2, 3, 128
+    q, dO = (_gen((B, N, Sq, D), s, dtype) for s in (301, 304))
+    k, v = (_gen((B, N, Sk, D), s, dtype) for s in (302, 303))
+    okw = dict(scale=D ** -0.5)
+    kw = {}
+    if causal:
+        okw.update(attn_mask=np.triu(np.ones((1, Sq, Sk), np.uint8), 1))
+        kw.update(mask_kind=_capi.MASK_CAUSAL)
+    tol = (ATOL, RTOL) if dtype == torch.float16 else (ATOL_BF16, RTOL_BF16)
+    _check_all(q, k, v, dO, okw, _run(q, k, v, dO, scale=D ** -0.5, **kw), *tol)
+
+
+def test_dq_kernel_with_64_rows_per_wave_on_bsnd_views():
+    B, N, S, D = 2, 4, 512, 128
+    store = [_gen((B, S, N, D), s).to(DEV) for s in (311, 312, 313, 314)]
+    q, k, v, dO = (t.permute(0, 2, 1, 3) for t in store)
+    tri = np.triu(np.ones((1, S, S), np.uint8), 1)
+    p = _capi.make_params(q, k, v, scale=D ** -0.5, mask_kind=_capi.MASK_CAUSAL)
+    o, lse = _capi.fa_fwd(p, q)
+    grads = _capi.fa_bwd(p, q, k, v, o, dO.contiguous(), lse)
+    torch.cuda.synchronize()
+    _check_all(q.cpu(), k.cpu(), v.cpu(), dO.cpu(), dict(scale=D ** -0.5, attn_mask=tri), (o, lse, grads))
+
+
 @pytest.mark.parametrize("D", [64, 80])
 def test_bf16_backward_at_the_small_head_dims(D):
     B, N, S = 2, 2, 300
