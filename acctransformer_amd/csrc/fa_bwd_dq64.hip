@@ -5,10 +5,11 @@
 // query rows of one (batch, head) and streams K/V tiles of 64 keys through LDS.  Here the workgroup is 4 waves
 // of 64 rows -- one wave per SIMD, 512 registers each -- instead of 8 waves of 32 rows: every K, V and K^T
 // fragment read from LDS feeds two MFMAs, which halves the LDS bytes per flop, the largest cost above the
-// matrix work in that kernel.  A lone wave per SIMD has no partner to overlap with, so the tile body is one
-// block of hand-scheduled assembly (fa_bwd_dq64_asm.inc, written by gen_dq64_asm.py) that threads the vector
-// work of one 32-key chunk between the MFMAs of the next; the accumulators and the Q / dO fragments live in
-// AGPRs at fixed registers.  The code around the block (prologue, tile DMA, barriers, epilogue) is HIP.
+// matrix work in that kernel.  A lone wave per SIMD has no partner to overlap with, so the tile loop is one
+// block of hand-scheduled assembly (fa_bwd_dq64_asm.inc, written by gen_dq64_asm.py), software-pipelined three
+// 32-key chunks deep: the vector work of one chunk rides behind the MFMAs of the score products of the next
+// and of the dQ product of the one before; the accumulators and the Q / dO fragments live in AGPRs at fixed
+// registers.  The code around the loop (prologue with the first two tiles' DMA, epilogue) is HIP.
 //
 // Served cases: head dim 128 exactly, no bias, no dropout, no mask tensor (mask none or the causal mask by
 // index compare), no row-block prefix, the band open towards earlier keys, Sq a multiple of 256 and Sk of 64.
@@ -34,17 +35,15 @@ template <typename T> struct Dq64Asm;
                : "{a[128:159]}"(qa), "{a[160:191]}"(qb), "{a[192:223]}"(doa), "{a[224:255]}"(dob), "{v[96:103]}"(koff), \
                  "{v[104:107]}"(toff), "{v108}"(nlq0), "{v109}"(nlq1), "{v110}"(dl0), "{v111}"(dl1),                      \
                  "{v[116:119]}"(kvoff), "{v[120:123]}"(vvoff), "{v124}"(rowrel0), "{v125}"(rowrel1),                      \
-                 [kbuf0] "s"(s.kbuf0), [ldssum] "s"(s.ldssum), [lds0] "s"(s.lds0), [kptr] "s"(s.kptr), [vptr] "s"(s.vptr), \
-                 [kstep] "s"(s.kstep), [vstep] "s"(s.vstep), [jhi] "s"(s.jhi), [wq0] "s"(s.wq0), [wq0p63] "s"(s.wq0p63),  \
-                 [causal] "s"(s.causal), [scale] "s"(s.scale)                                                            \
+                 [kbuf0] "s"(s.kbuf0), [lds0] "s"(s.lds0), [kptr] "s"(s.kptr), [vptr] "s"(s.vptr), [kstep] "s"(s.kstep),       \
+                 [vstep] "s"(s.vstep), [jhi] "s"(s.jhi), [jlast] "s"(s.jlast), [lastedge] "s"(s.lastedge), [scale] "s"(s.scale) \
                : DQ64_CLOBBERS)
 struct Dq64Scalars {
-  uint32_t kbuf0, ldssum, lds0;      // LDS: first K tile buffer, sum of the two buffers' addresses, this wave's slab inside a tile
-  uint64_t kptr, vptr;               // global address of the K / V rows of tile 1 (tile 0 when there is no other)
+  uint32_t kbuf0, lds0;              // LDS: first of the three K/V tile buffers, this wave's slab inside a tile
+  uint64_t kptr, vptr;               // global address of the K / V rows of tile 2 (of the last tile when there are fewer)
   uint32_t kstep, vstep;             // bytes from one tile's rows to the next
-  uint32_t jhi;                      // last tile
-  int32_t wq0, wq0p63;               // first and last query row of the wave
-  uint32_t causal;
+  uint32_t jhi;                      // last tile of the workgroup
+  uint32_t jlast, lastedge;          // last tile of this wave; whether the causal diagonal runs through it
   float scale;                       // scale * log2(e)
 };
 template <> struct Dq64Asm<f16> {
@@ -71,7 +70,7 @@ __global__ void __launch_bounds__(256) fa_bwd_dq64_kernel(const FaArgs a) {
   using C = SwzCfg<D>;
   constexpr int TILEB = 64 * C::PITCH;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [2 buffers][K tile | V tile]; reused by the epilogue
+  ACCT_LDS char* smem = (ACCT_LDS char*)smem_raw;   // [3 buffers][K tile | V tile]; reused by the epilogue
 
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -144,27 +143,28 @@ __global__ void __launch_bounds__(256) fa_bwd_dq64_kernel(const FaArgs a) {
   kdma.plan(a.k_ss, D / 8);
   vdma.plan(a.v_ss, D / 8);
   if (j_lo <= j_hi) {
-    kdma.issue(kp, a.k_ss, j_lo * 64, smem);
-    vdma.issue(vp, a.v_ss, j_lo * 64, smem + TILEB);
-    // tile 0 has landed before the loop starts; inside it every tile is requested one step ahead
+    // tiles 0 and 1 have landed before the loop starts; inside it every tile is requested two steps ahead
+    const int t1 = min(1, j_hi) * 64, t2 = min(2, j_hi) * 64;
+    kdma.issue(kp, a.k_ss, 0, smem);
+    vdma.issue(vp, a.v_ss, 0, smem + TILEB);
+    kdma.issue(kp, a.k_ss, t1, smem + 2 * TILEB);
+    vdma.issue(vp, a.v_ss, t1, smem + 3 * TILEB);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     auto uniform = [](uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); };
     Dq64Scalars s;
     s.kbuf0 = uniform((uint32_t)(uintptr_t)smem);
-    s.ldssum = uniform(2 * (uint32_t)(uintptr_t)smem + 2 * TILEB);
     s.lds0 = uniform(kdma.lds0);
-    // (rows of tile 1, the first one the loop requests; with a single tile it is requested once more instead)
-    const int t1 = j_hi > 0 ? 64 : 0;
-    const uint64_t kptr = (uint64_t)(uintptr_t)(kp + (int64_t)t1 * a.k_ss), vptr = (uint64_t)(uintptr_t)(vp + (int64_t)t1 * a.v_ss);
+    const uint64_t kptr = (uint64_t)(uintptr_t)(kp + (int64_t)t2 * a.k_ss), vptr = (uint64_t)(uintptr_t)(vp + (int64_t)t2 * a.v_ss);
     s.kptr = ((uint64_t)uniform((uint32_t)(kptr >> 32)) << 32) | uniform((uint32_t)kptr);
     s.vptr = ((uint64_t)uniform((uint32_t)(vptr >> 32)) << 32) | uniform((uint32_t)vptr);
     s.kstep = uniform((uint32_t)(64 * a.k_ss * (int64_t)sizeof(T)));
     s.vstep = uniform((uint32_t)(64 * a.v_ss * (int64_t)sizeof(T)));
     s.jhi = uniform((uint32_t)j_hi);
-    s.wq0 = (int32_t)uniform((uint32_t)wq0);
-    s.wq0p63 = s.wq0 + 63;
-    s.causal = uniform(causal ? 1u : 0u);
+    // under the causal mask the wave's 64 rows end with the 64 keys of tile wq0 / 64, if the keys reach that far
+    const int jdiag = wq0 / 64;
+    s.jlast = uniform((uint32_t)(causal ? min(jdiag, j_hi) : j_hi));
+    s.lastedge = uniform(causal && jdiag <= j_hi ? 1u : 0u);
     s.scale = a.scale_log2e;
     const u32x4 kvoff = {kdma.voff[0], kdma.voff[1], kdma.voff[2], kdma.voff[3]};
     const u32x4 vvoff = {vdma.voff[0], vdma.voff[1], vdma.voff[2], vdma.voff[3]};
@@ -207,7 +207,7 @@ bool dq64_applicable(const FaArgs& a) {
 }
 
 hipError_t launch_bwd_dq64(FaArgs a, int dtype, hipStream_t st) {
-  constexpr size_t smem = 4 * 64 * 256;               // two K/V tile pairs (the epilogue's transposition fits inside)
+  constexpr size_t smem = 6 * 64 * 256;               // three K/V tile pairs (the epilogue's transposition fits inside)
   a.n_tiles = a.Sq / 256;
   const dim3 grid((unsigned)((long long)a.n_tiles * a.B * a.N));
   hipError_t e;
