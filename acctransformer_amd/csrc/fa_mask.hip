@@ -217,19 +217,42 @@ hipError_t launch_mask_colbits(const FaArgs& a, const uint8_t* flags, uint32_t* 
   return hipGetLastError();
 }
 
+// Column entries of the dropout bitmaps, written whole.  The four waves of a workgroup each hold, per lane and for
+// sixteen keys, the 32-bit word of their 32 rows; a key's 16-byte entry is the four waves' words.  Written straight
+// from the waves every entry would be four 4-byte stores from four places; instead the words cross LDS and every
+// thread stores complete entries, consecutive threads consecutive entries.  key_of(lane, e): the key of a lane's
+// e-th word.  (One spare entry after every sixteen keeps the word stores of a wave on different banks.)
+template <typename KeyOf>
+ACCT_DEV void store_col_entries(uint32_t* s_cw, const uint32_t (&cw)[16], int wave, int lane, int key0, int Sk, uint32_t* out,
+                                KeyOf key_of) {
+#pragma unroll
+  for (int e = 0; e < 16; e++) {
+    const int k = key_of(lane, e);                       // 0 .. 1023 within the span
+    s_cw[(k + (k >> 4)) * 4 + wave] = __builtin_bitreverse32(cw[e]);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int m = 0; m < 4; m++) {
+    const int k = threadIdx.x + 256 * m;
+    if (key0 + k < Sk)
+      *reinterpret_cast<u32x4*>(out + (int64_t)(key0 + k) * 4) = *reinterpret_cast<const u32x4*>(s_cw + (k + (k >> 4)) * 4);
+  }
+}
+
 // Dropout mask (uint8 {0,1}, or the reference's {0, 1/keep_prob} in the I/O dtype; nonzero = keep) packed into keep bits, by query row for the kernels whose lanes own
-// query rows (forward, dQ) and by key column for the dK/dV kernel.  One wave per (batch*head, 32 query
-// rows, 1024 keys) -- enough waves to keep the memory system busy --: per row every lane loads the 16 bytes of keys 16*lane .. +15 (a kilobyte per wave
+// query rows (forward, dQ) and by key column for the dK/dV kernel.  One workgroup of four waves per (batch*head,
+// 128 query rows, 1024 keys), one wave per 32 rows -- enough waves to keep the memory system busy --: per row every lane loads the 16 bytes of keys 16*lane .. +15 (a kilobyte per wave
 // instruction keeps enough bytes in flight) and turns them into 16 bits; lane pairs form the 32-bit row words.
 //   rowbits [B*N*Sq, 2*ceil(Sk/64)] 32-bit: bit k of word w = keep[row][32w + k];
 //   colbits [B*N, Tr, Sk, 4] 32-bit: bit r of the 128-bit entry = keep[128*qb + r][key].
 template <int ES>
-__global__ void __launch_bounds__(64) fa_drop_bits_kernel(const FaArgs a, uint32_t* rowbits, uint32_t* colbits) {
+__global__ void __launch_bounds__(256) fa_drop_bits_kernel(const FaArgs a, uint32_t* rowbits, uint32_t* colbits) {
+  __shared__ __attribute__((aligned(16))) uint32_t s_cw[(1024 + 64) * 4];
   const int nspan = (a.Sk + 1023) / 1024;
-  const int i = blockIdx.x & 3;                         // which 32 rows of the 128-row block: word i of the column entries
-  const int blk = blockIdx.x >> 2;
+  const int i = threadIdx.x >> 6;                       // which 32 rows of the 128-row block: word i of the column entries
+  const int blk = blockIdx.x;
   const int span = blk % nspan, qb = (blk / nspan) % a.Tr, bh = blk / (nspan * a.Tr);
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63;
   const int kv = span * 1024 + 16 * lane;               // first of this lane's sixteen keys
   const bool vec = (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 15) == 0 && kv + 16 <= a.Sk;   // (16 elements: ES aligned 16-byte loads)
   // Keys in a block that the attention mask's pre-pass classed 'skip' are never visited by the attention kernels:
@@ -282,24 +305,24 @@ __global__ void __launch_bounds__(64) fa_drop_bits_kernel(const FaArgs a, uint32
       rowout += a.droprow_w;
     }
   }
-  if (colbits) {
-#pragma unroll
-    for (int e = 0; e < 16; e++)
-      if (kv + e < a.Sk) colbits[(((int64_t)bh * a.Tr + qb) * a.Sk + kv + e) * 4 + i] = __builtin_bitreverse32(cw[e]);
-  }
+  if (colbits)
+    store_col_entries(s_cw, cw, i, lane, span * 1024, a.Sk, colbits + ((int64_t)bh * a.Tr + qb) * a.Sk * 4,
+                      [](int l, int e) { return 16 * l + e; });
 }
 
 // The same bitmaps for counter-based dropout: nothing is read, the keep decisions come from Philox4x32-10.
 // One call yields the 16 bytes of one (query row, 32-key group M, half g): keys 32M + 8u + 4g + e for
 // u = 0..3, e = 0..3 -- the keys one lane of the attention kernels owns in a 32-key group, so a kernel
-// could also draw them in place.  One wave per (batch*head, 32 query rows, 1024 keys); lane 2L + g owns
+// could also draw them in place.  One workgroup of four waves per (batch*head, 128 query rows, 1024 keys), one
+// wave per 32 rows; lane 2L + g owns
 // (M = 32*span + L, g), the lane pair forms the 32-bit row word of group M.
-__global__ void __launch_bounds__(64) fa_drop_philox_kernel(const FaArgs a, uint32_t* rowbits, uint32_t* colbits) {
+__global__ void __launch_bounds__(256) fa_drop_philox_kernel(const FaArgs a, uint32_t* rowbits, uint32_t* colbits) {
+  __shared__ __attribute__((aligned(16))) uint32_t s_cw[(1024 + 64) * 4];
   const int nspan = (a.Sk + 1023) / 1024;
-  const int i = blockIdx.x & 3;                         // which 32 rows of the 128-row block: word i of the column entries
-  const int blk = blockIdx.x >> 2;
+  const int i = threadIdx.x >> 6;                       // which 32 rows of the 128-row block: word i of the column entries
+  const int blk = blockIdx.x;
   const int span = blk % nspan, qb = (blk / nspan) % a.Tr, bh = blk / (nspan * a.Tr);
-  const int lane = threadIdx.x, g = lane & 1;
+  const int lane = threadIdx.x & 63, g = lane & 1;
   const int grp = 32 * span + (lane >> 1);              // 32-key group = word index within the row
   const bool writer = rowbits && g == 0 && grp < a.droprow_w;
   uint32_t* rowout = rowbits + ((int64_t)bh * a.Sq + qb * 128 + 32 * i) * a.droprow_w + grp;
@@ -326,25 +349,21 @@ __global__ void __launch_bounds__(64) fa_drop_philox_kernel(const FaArgs a, uint
       rowout += a.droprow_w;
     }
   }
-  if (colbits) {
-#pragma unroll
-    for (int t = 0; t < 16; t++) {
-      const int key = 32 * grp + 8 * (t >> 2) + 4 * g + (t & 3);
-      if (key < a.Sk) colbits[(((int64_t)bh * a.Tr + qb) * a.Sk + key) * 4 + i] = __builtin_bitreverse32(cw[t]);
-    }
-  }
+  if (colbits)
+    store_col_entries(s_cw, cw, i, lane, span * 1024, a.Sk, colbits + ((int64_t)bh * a.Tr + qb) * a.Sk * 4,
+                      [](int l, int t) { return 32 * (l >> 1) + 8 * (t >> 2) + 4 * (l & 1) + (t & 3); });
 }
 
 hipError_t launch_drop_philox(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st) {
-  const long long nblk = 4LL * a.B * a.N * a.Tr * ((a.Sk + 1023) / 1024);
-  hipLaunchKernelGGL(fa_drop_philox_kernel, dim3((unsigned)nblk), dim3(64), 0, st, a, rowbits, colbits);
+  const long long nblk = (long long)a.B * a.N * a.Tr * ((a.Sk + 1023) / 1024);
+  hipLaunchKernelGGL(fa_drop_philox_kernel, dim3((unsigned)nblk), dim3(256), 0, st, a, rowbits, colbits);
   return hipGetLastError();
 }
 
 hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st) {
-  const long long nblk = 4LL * a.B * a.N * a.Tr * ((a.Sk + 1023) / 1024);
-  if (a.drop_es == 2) hipLaunchKernelGGL(fa_drop_bits_kernel<2>, dim3((unsigned)nblk), dim3(64), 0, st, a, rowbits, colbits);
-  else hipLaunchKernelGGL(fa_drop_bits_kernel<1>, dim3((unsigned)nblk), dim3(64), 0, st, a, rowbits, colbits);
+  const long long nblk = (long long)a.B * a.N * a.Tr * ((a.Sk + 1023) / 1024);
+  if (a.drop_es == 2) hipLaunchKernelGGL(fa_drop_bits_kernel<2>, dim3((unsigned)nblk), dim3(256), 0, st, a, rowbits, colbits);
+  else hipLaunchKernelGGL(fa_drop_bits_kernel<1>, dim3((unsigned)nblk), dim3(256), 0, st, a, rowbits, colbits);
   return hipGetLastError();
 }
 
