@@ -248,66 +248,80 @@ ACCT_DEV void store_col_entries(uint32_t* s_cw, const uint32_t (&cw)[16], int wa
 template <int ES>
 __global__ void __launch_bounds__(256) fa_drop_bits_kernel(const FaArgs a, uint32_t* rowbits, uint32_t* colbits) {
   __shared__ __attribute__((aligned(16))) uint32_t s_cw[(1024 + 64) * 4];
+  // A lane's sixteen keys of the span come from ES 16-byte loads of 16 / ES keys each; load h of the wave reads one
+  // contiguous kilobyte: keys 16*lane + e for bytes, keys 512 h + 8*lane + e for 2-byte elements.
+  constexpr int NH = ES, KH = 16 / ES;
   const int nspan = (a.Sk + 1023) / 1024;
   const int i = threadIdx.x >> 6;                       // which 32 rows of the 128-row block: word i of the column entries
   const int blk = blockIdx.x;
   const int span = blk % nspan, qb = (blk / nspan) % a.Tr, bh = blk / (nspan * a.Tr);
   const int lane = threadIdx.x & 63;
-  const int kv = span * 1024 + 16 * lane;               // first of this lane's sixteen keys
-  const bool vec = (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 15) == 0 && kv + 16 <= a.Sk;   // (16 elements: ES aligned 16-byte loads)
+  const bool aligned = (((uintptr_t)a.drop | (uintptr_t)a.Sk) & 15) == 0;     // (16 elements: aligned 16-byte loads)
   // Keys in a block that the attention mask's pre-pass classed 'skip' are never visited by the attention kernels:
   // their keep bits are not read, so their mask bytes are not loaded either (this pass is bound by the bytes it
   // reads; a padded batch skips a third to a half of them).
-  const bool dead = a.blkflags && kv < a.Sk &&
-                    a.blkflags[((int64_t)(a.mask_sb ? bh / a.N : 0) * a.Tr + qb) * a.Tc + kv / 128] == kBlkSkip;
-  const int widx = 32 * span + (lane >> 1);             // this lane pair's word within the row
-  const bool writer = rowbits && (lane & 1) == 0 && widx < a.droprow_w;
+  const uint8_t* flags = a.blkflags ? a.blkflags + ((int64_t)(a.mask_sb ? bh / a.N : 0) * a.Tr + qb) * a.Tc : nullptr;
+  int kv[NH];                                           // first key of each load
+  bool vec[NH], dead[NH];
+  const uint8_t* p[NH];
+#pragma unroll
+  for (int h = 0; h < NH; h++) {
+    kv[h] = span * 1024 + (ES == 1 ? 16 * lane : 512 * h + 8 * lane);
+    vec[h] = aligned && kv[h] + KH <= a.Sk;
+    dead[h] = kv[h] >= a.Sk || (flags && flags[kv[h] / 128] == kBlkSkip);
+    p[h] = a.drop + (((int64_t)bh * a.Sq + qb * 128 + 32 * i) * a.Sk + min(kv[h], max(a.Sk - KH, 0))) * ES;
+  }
+  // row words: 32 keys are two lanes' bits for bytes, four lanes' for 2-byte elements (whose second load fills
+  // the words sixteen further on)
+  constexpr int LPW = 32 / KH;                          // lanes per word
+  const int widx = 32 * span + lane / LPW;
+  const bool writer = rowbits && lane % LPW == 0;
   uint32_t* rowout = rowbits + ((int64_t)bh * a.Sq + qb * 128 + 32 * i) * a.droprow_w + widx;
-  const uint8_t* p = a.drop + (((int64_t)bh * a.Sq + qb * 128 + 32 * i) * a.Sk + min(kv, max(a.Sk - 16, 0))) * ES;
   const int nrow = min(128, a.Sq - qb * 128);
   uint32_t cw[16];                                      // per key: the word of these 32 rows, most significant bit first
-  {
 #pragma unroll
-    for (int e = 0; e < 16; e++) cw[e] = 0u;
+  for (int e = 0; e < 16; e++) cw[e] = 0u;
 #pragma unroll 16
-    for (int r = 0; r < 32; r++) {
-      const int rr = 32 * i + r;
-      uint32_t nz = 0;                                  // bit e: this lane's key e of the row is kept
-      if (rr < nrow && !dead) {
-        if (vec) {
+  for (int r = 0; r < 32; r++) {
+    const int rr = 32 * i + r;
+    uint32_t nz = 0;                                    // bit KH*h + e: key e of this lane's load h is kept
 #pragma unroll
-          for (int h = 0; h < ES; h++) {
-            const u32x4 v = *reinterpret_cast<const u32x4*>(p + 16 * h);
+    for (int h = 0; h < NH; h++) {
+      if (rr < nrow && !dead[h]) {
+        if (vec[h]) {
+          const u32x4 v = *reinterpret_cast<const u32x4*>(p[h]);
 #pragma unroll
-            for (int w = 0; w < 4; w++) {
-              if (ES == 1) {
+          for (int w = 0; w < 4; w++) {
+            if (ES == 1) {
 #pragma unroll
-                for (int e = 0; e < 4; e++) nz |= (((v[w] >> (8 * e)) & 0xffu) != 0 ? 1u : 0u) << (4 * w + e);
-              } else {
-                nz |= (((v[w] & 0x7fffu) != 0 ? 1u : 0u) | (((v[w] >> 16) & 0x7fffu) != 0 ? 2u : 0u)) << (8 * h + 2 * w);
-              }
+              for (int e = 0; e < 4; e++) nz |= (((v[w] >> (8 * e)) & 0xffu) != 0 ? 1u : 0u) << (4 * w + e);
+            } else {
+              nz |= (((v[w] & 0x7fffu) != 0 ? 1u : 0u) | (((v[w] >> 16) & 0x7fffu) != 0 ? 2u : 0u)) << (KH * h + 2 * w);
             }
           }
         } else {
           const uint8_t* q = a.drop + ((int64_t)bh * a.Sq + qb * 128 + rr) * a.Sk * ES;
 #pragma unroll
-          for (int e = 0; e < 16; e++)
-            if (kv + e < a.Sk && elem_nonzero<ES>(q, kv + e)) nz |= 1u << e;
+          for (int e = 0; e < KH; e++)
+            if (kv[h] + e < a.Sk && elem_nonzero<ES>(q, kv[h] + e)) nz |= 1u << (KH * h + e);
         }
       }
-      p += (int64_t)a.Sk * ES;                          // per-lane pointer walks down the rows
-      const uint32_t bits = nz;
-#pragma unroll
-      for (int e = 0; e < 16; e++) cw[e] = (cw[e] << 1) | ((nz >> e) & 1u);
-      uint32_t x = bits << (16 * (lane & 1));
-      x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xf, 0xf, true);    // lane ^ 1
-      if (writer && rr < nrow) *rowout = x;
-      rowout += a.droprow_w;
+      p[h] += (int64_t)a.Sk * ES;                       // per-lane pointers walk down the rows
     }
+#pragma unroll
+    for (int e = 0; e < 16; e++) cw[e] = (cw[e] << 1) | ((nz >> e) & 1u);
+#pragma unroll
+    for (int h = 0; h < NH; h++) {
+      uint32_t x = ((nz >> (KH * h)) & ((1u << KH) - 1u)) << (KH * (lane % LPW));
+      x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xf, 0xf, true);                   // lane ^ 1
+      if (LPW == 4) x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xf, 0xf, true);     // lane ^ 2
+      if (writer && rr < nrow && widx + 16 * h < a.droprow_w) rowout[16 * h] = x;
+    }
+    rowout += a.droprow_w;
   }
   if (colbits)
     store_col_entries(s_cw, cw, i, lane, span * 1024, a.Sk, colbits + ((int64_t)bh * a.Tr + qb) * a.Sk * 4,
-                      [](int l, int e) { return 16 * l + e; });
+                      [](int l, int e) { return ES == 1 ? 16 * l + e : 512 * (e >> 3) + 8 * l + (e & 7); });
 }
 
 // The same bitmaps for counter-based dropout: nothing is read, the keep decisions come from Philox4x32-10.
