@@ -858,7 +858,7 @@ def _random_case(rng):
     """One random configuration of the operator: shapes, element type, mask form, band, bias form, dropout form,
     memory layout.  Small enough for the fp64 oracle; every option the C ABI has can come up with every other."""
     D = int(rng.choice([8, 24, 40, 64, 72, 80, 96, 128, 160, 200, 256]))
-    side_ok = D != 40 and D <= 128                       # bias and dropout variants exist for these head dims
+    bias_ok = D != 40 and D <= 128                       # bias variants exist for these head dims (dropout for all)
     B, N = int(rng.integers(1, 3)), int(rng.integers(1, 4))
     if rng.random() < 0.5:
         Sq = Sk = int(rng.choice([64, 128, 200, 256, 333, 384, 520]))
@@ -875,8 +875,8 @@ def _random_case(rng):
         c["prev"], c["nxt"] = int(rng.choice([0, 1, 2, 65536])), int(rng.choice([0, 1, 65536]))
     if c["mask"] == "tile":
         c["nxt"] = 0
-    c["bias"] = str(rng.choice(["none", "row", "row_batched", "full"])) if side_ok and rng.random() < 0.5 else "none"
-    c["drop"] = str(rng.choice(["u8", "f16", "seed"])) if side_ok and rng.random() < 0.4 else "none"
+    c["bias"] = str(rng.choice(["none", "row", "row_batched", "full"])) if bias_ok and rng.random() < 0.5 else "none"
+    c["drop"] = str(rng.choice(["u8", "f16", "seed"])) if rng.random() < 0.4 else "none"
     return c
 
 
@@ -933,6 +933,58 @@ def test_random_configurations_against_oracle(block):
             _check_all(q, k, v, dO, okw, _run(q, k, v, dO, **kw), saved_o=True, **tol)
         except AssertionError as e:
             raise AssertionError(f"{c}: {e}") from e
+
+
+@pytest.mark.parametrize("D", [8, 24, 72, 200])
+def test_one_to_fifteen_keys_with_side_inputs(D):
+    # The random sweep above draws at least 16 keys.  Below that dV and dK have nothing to average over: an entry
+    # sums Sq products P*dO (dV) or scale*dS*q (dK) whose P, dS (of order 1, not 1/Sk) are rounded to the I/O type
+    # before the product, relative error u = 2^-11 (fp16), uniformly distributed, so the entry's error has standard
+    # deviation <= u/sqrt(3) * sqrt(sum dO^2) ~ u/sqrt(3) * sqrt(Sq) for N(0,1) operands whatever the entry's own
+    # size.  The gate for dV and dK is therefore widened by four such standard deviations (over keep_prob with
+    # dropout).  dQ sums Sk products scale*dS*k: dP = dO.v has standard deviation sqrt(D) = 1/scale, so scale*dS is
+    # of order 1/keep_prob with tails to three times that, rounded with the same u: four standard deviations of
+    # that sum are added to its gate.  O keeps the acceptance gate.
+    rng = np.random.default_rng(4100 + D)
+    u = 2.0 ** -11
+    n = 0
+    for Sk in (1, 2, 3, 7, 15):
+        for Sq in (40, 333):
+            B, N = 2, 2
+            q, dO = (_gen((B, N, Sq, D), int(s)) for s in rng.integers(1, 1 << 30, size=2))
+            k, v = (_gen((B, N, Sk, D), int(s)) for s in rng.integers(1, 1 << 30, size=2))
+            scale = D ** -0.5
+            kw, okw = dict(scale=scale), dict(scale=scale)
+            mask = ("none", "causal", "dense_random")[n % 3]
+            if mask == "causal":
+                kw.update(mask_kind=_capi.MASK_CAUSAL); okw.update(attn_mask=np.triu(np.ones((1, Sq, Sk), np.uint8), 1))
+            elif mask == "dense_random":
+                m = (rng.random((B, Sq, Sk)) < 0.3).astype(np.uint8); m[:, :, 0] = 0
+                kw.update(mask_kind=_capi.MASK_DENSE_U8, attn_mask=m); okw.update(attn_mask=m)
+            if D <= 128 and n % 2 == 0:                  # (bias variants exist up to head dim 128)
+                al = (0.3 * torch.randn((1, N, 1, Sk) if n % 4 == 0 else (1, N, Sq, Sk), generator=torch.Generator().manual_seed(n))).half()
+                kw.update(alibi=al); okw.update(alibi=al.float().numpy())
+            if n % 3 != 1:
+                keep = (0.9, 0.5)[n % 2]
+                if n % 5 < 3:
+                    seed, off = (977 + n) << 20, n
+                    kw.update(keep_prob=keep, drop_seed=seed, drop_offset=off)
+                    okw.update(drop_mask=phx.dropout_keep_mask(B, N, Sq, Sk, seed, off, keep), keep_prob=phx.keep_threshold(keep) / 256.0)
+                else:
+                    drop = (rng.random((B, N, Sq, Sk)) < keep).astype(np.uint8)
+                    kw.update(keep_prob=keep, drop_mask=drop); okw.update(drop_mask=drop, keep_prob=keep)
+            o, lse, grads = _run(q, k, v, dO, **kw)
+            f = _np
+            O, L = orc.unfused_fwd(f(q), f(k), f(v), **okw)
+            dQ, dK, dV = orc.unfused_bwd(f(q), f(k), f(v), f(dO), **okw, O_saved=_np(o))
+            what = f"D={D} Sq={Sq} Sk={Sk} mask={mask} case {n}"
+            _gate(O, o, what=what + " O")
+            kp = okw.get("keep_prob", 1.0)
+            _gate(dQ, grads[0], atol=ATOL + 4 * u / 3 ** 0.5 * Sk ** 0.5 * 3 / kp, what=what + " dQ")
+            wide = ATOL + 4 * u / 3 ** 0.5 * Sq ** 0.5 / kp
+            _gate(dK, grads[1], atol=wide, what=what + " dK")
+            _gate(dV, grads[2], atol=wide, what=what + " dV")
+            n += 1
 
 
 @pytest.mark.parametrize("block", range(3))
