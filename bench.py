@@ -475,7 +475,7 @@ def main():
     }
     # HBM-side bytes per launch, from the FETCH_SIZE / WRITE_SIZE counter runs summarised under profiles/
     # (each scaled by what the same counter reads for a 256 MiB copy kernel: x2.000 and x1.000)
-    traffic_bytes = {"fa_fwd_kernel": 194.0e6, "fa_bwd_dq_kernel": 308.7e6, "fa_bwd_dkdv_kernel": 287.5e6}
+    traffic_bytes = {"fa_fwd_kernel": 189.5e6, "fa_bwd_dq_kernel": 292.7e6, "fa_bwd_dkdv_kernel": 287.1e6}
     dom = max(kernels, key=lambda n: kernels[n][0])
     dom_ms, dom_fl = kernels[dom]
     achieved = dom_fl / (dom_ms * 1e-3) / 1e12
