@@ -203,7 +203,9 @@ __global__ void __launch_bounds__(256) fa_bwd_dq64_kernel(const FaArgs a) {
 bool dq64_applicable(const FaArgs& a) {
   const bool no_side = !a.alibi && !a.droprow && !a.dropcol && (a.mask_kind == kMaskNone || a.mask_kind == kMaskCausal);
   const bool band_open = a.prev_blk >= a.Tr && (a.mask_kind == kMaskCausal || a.next_blk >= a.Tc);
-  return no_side && band_open && a.hd == 128 && a.row_prefix == 0 && a.Sq % 256 == 0 && a.Sk % 64 == 0;
+  // (the loop advances its tile addresses by 32-bit byte steps)
+  const bool steps_fit = a.k_ss < (1 << 23) && a.v_ss < (1 << 23);
+  return no_side && band_open && steps_fit && a.hd == 128 && a.row_prefix == 0 && a.Sq % 256 == 0 && a.Sk % 64 == 0;
 }
 
 hipError_t launch_bwd_dq64(FaArgs a, int dtype, hipStream_t st) {
