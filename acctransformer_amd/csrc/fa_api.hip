@@ -231,11 +231,14 @@ acct::FaArgs make_args(const acct_fa_params* p) {
   return a;
 }
 
-// block classes of a dense mask: one byte per 128x128 block
+// block classes of a dense mask, one byte per 128x128 block, followed by the key-tail table of the same size
+size_t class_count(const acct_fa_params* p) {
+  const size_t MB = p->mask_stride_b ? p->B : 1;
+  return MB * (size_t)((p->Sq + 127) / 128) * (size_t)((p->Sk + 127) / 128);
+}
 size_t flag_bytes(const acct_fa_params* p) {
   if (!mask_is_dense(p)) return 0;
-  const size_t MB = p->mask_stride_b ? p->B : 1;
-  return align_up(MB * (size_t)((p->Sq + 127) / 128) * (size_t)((p->Sk + 127) / 128), 256);
+  return align_up(2 * class_count(p), 256);
 }
 
 // per-key-column bitmaps of the mixed blocks of a dense mask (backward only): 16 bytes per (q block, key)
@@ -269,7 +272,12 @@ int mask_prepass(acct::FaArgs& a, const acct_fa_params* p, uint8_t* own, bool wa
   uint32_t* cbits = (uint32_t*)(base + flag_bytes(p));
   const bool filled = p->mask_bits && p->mask_bits_filled;
   const bool cols = p->mask_bits ? true : want_cols;
-  if (mask_is_dense(p)) a.blkflags = flags;
+  if (mask_is_dense(p)) {
+    a.blkflags = flags;
+    // (only the one-launch pre-pass writes the key tails; which path runs follows from the arguments alone, so every
+    // call of a step that shares a mask_bits buffer decides alike)
+    a.blktail = acct::mask_prepass_is_fused(a) ? flags + class_count(p) : nullptr;
+  }
   if (cols) a.colbits = cbits;
   if (filled) return ACCT_OK;
   hipError_t e = mask_is_dense(p) ? acct::launch_mask_blocks(a, flags, cols ? cbits : nullptr, p->mask_stride_b ? p->B : 1, st)

@@ -77,7 +77,8 @@ ACCT_DEV void fa_bwd_dq_body(const FaArgs& a) {
     // band, one round trip to memory yields both the trimmed range and the wave's class window.
     const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc;
     int b_lo = j_lo >> 1, b_hi = j_hi >> 1;
-    if (j_lo <= j_hi && flwin.init_trimmed(fl, 1, a.Tc, qb_lo, qb_hi - qb_lo + 1, min(wqb, qb_hi), b_lo, b_hi, lane)) {
+    const uint8_t* tails = a.blktail ? a.blktail + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc : nullptr;
+    if (j_lo <= j_hi && flwin.init_trimmed(fl, 1, a.Tc, qb_lo, qb_hi - qb_lo + 1, min(wqb, qb_hi), b_lo, b_hi, lane, tails)) {
       j_lo = max(j_lo, b_lo * 2);
       j_hi = min(j_hi, b_hi * 2 + 1);
       flwin_ready = true;
@@ -185,7 +186,7 @@ ACCT_DEV void fa_bwd_dq_body(const FaArgs& a) {
 
     // block classes of a dense mask: 64 blocks at a time into scalar registers
     const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
-    if (!flwin_ready) flwin.init(flrow, 1, j_lo >> 1, j_hi >> 1, lane);
+    if (!flwin_ready) flwin.init(flrow, 1, j_lo >> 1, j_hi >> 1, lane, (flrow && a.blktail) ? a.blktail + (flrow - a.blkflags) : nullptr);
     for (int j = j_lo; j <= j_hi; j++) {
       const uint32_t fl_cur = flwin.get(j >> 1, lane);
       const int buf = (j - j_lo) & 1;
@@ -209,14 +210,24 @@ ACCT_DEV void fa_bwd_dq_body(const FaArgs& a) {
       act = act && (kv0 < wkv_limit);
       bool apply_mask = false;
       bool diag = causal;                                   // keys after the query are hidden, by index compare
+      int last_key = a.Sk - 1;                              // last key that exists and is not behind a key tail
       if (MASKT && a.mask_kind == kMaskDense && act) {
         act = fl_cur != kBlkSkip;
         apply_mask = fl_cur == kBlkApply;
         if (fl_cur == kBlkTriu) { diag = true; act = kv0 <= wq_end - 1; }
+        if (apply_mask) {
+          const int tail = (int)flwin.tail(kvb);
+          if (tail) {
+            // every row of the block hides exactly the keys from its tail-th on: an index compare, no mask loads
+            apply_mask = false;
+            last_key = min(last_key, kvb * 128 + tail - 1);
+            act = kv0 <= last_key;
+          }
+        }
       } else if (MASKT && a.mask_kind == kMaskTile) {
         apply_mask = wqb == kvb;
       }
-      const bool edge = apply_mask || (diag && (kv0 + 63 > wq0)) || (kv0 + 64 > a.Sk);
+      const bool edge = apply_mask || (diag && (kv0 + 63 > wq0)) || (kv0 + 63 > last_key);
       if (act) {
         V8 dsf[QG][2][2];
 #pragma unroll
@@ -297,7 +308,7 @@ ACCT_DEV void fa_bwd_dq_body(const FaArgs& a) {
             } else if (!apply_mask && !bias_pending && !DROP) {
               // causal diagonal and/or ragged key tail only: P of a hidden key is exactly 0 (with the
               // additive mask it underflows to the same value), one compare and select per element
-              int vis = a.Sk - 1 - kv0 - 32 * c - 4 * g;         // last visible key, relative to this lane's first
+              int vis = last_key - kv0 - 32 * c - 4 * g;         // last visible key, relative to this lane's first
               if (diag) vis = min(vis, qrow - kv0 - 32 * c - 4 * g);
 #pragma unroll
               for (int r = 0; r < 16; r++) {
@@ -331,9 +342,9 @@ ACCT_DEV void fa_bwd_dq_body(const FaArgs& a) {
                     if ((mbits >> (8 * e)) & 0xffu) x[4 * r4 + e] += kMaskFill * kLog2e;
                 }
               }
-              if ((diag && (kv0 + 63 > wq0)) || (kv0 + 64 > a.Sk)) {
-                // keys after the query (causal) or past Sk: P is exactly 0
-                int vis = a.Sk - 1 - kv0 - 32 * c - 4 * g;
+              if ((diag && (kv0 + 63 > wq0)) || (kv0 + 63 > last_key)) {
+                // keys after the query (causal), past Sk or behind a key tail: P is exactly 0
+                int vis = last_key - kv0 - 32 * c - 4 * g;
                 if (diag) vis = min(vis, qrow - kv0 - 32 * c - 4 * g);
 #pragma unroll
                 for (int r = 0; r < 16; r++)
@@ -611,7 +622,9 @@ ACCT_DEV void fa_bwd_dkdv_body(const FaArgs& a) {
     // blocks, one round trip to memory yields both the trimmed range and the pair's class window.
     const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc;
     int b_lo = i_lo >> 1, b_hi = i_hi >> 1;
-    if (i_lo <= i_hi && flwin.init_trimmed(fl, a.Tc, 1, kb_lo, kb_hi - kb_lo + 1, min(wkb, kb_hi), b_lo, b_hi, lane)) {
+    // (the bias variants have no register to spare for the key tails: they read such blocks through the bitmaps)
+    const uint8_t* tails = (!BIAS && a.blktail) ? a.blktail + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc : nullptr;
+    if (i_lo <= i_hi && flwin.init_trimmed(fl, a.Tc, 1, kb_lo, kb_hi - kb_lo + 1, min(wkb, kb_hi), b_lo, b_hi, lane, tails)) {
       i_lo = max(i_lo, b_lo * 2);
       i_hi = min(i_hi, b_hi * 2 + 1);
       flwin_ready = true;
@@ -709,8 +722,9 @@ ACCT_DEV void fa_bwd_dkdv_body(const FaArgs& a) {
 
   // per-chunk predicates of this pair (chunk = 32 query rows; two per staged tile), as bits of one value
   // so that they live in a register: 1 act, 2 apply_mask, 4 limits (some (row, key) of the chunk is
-  // absent), 8 diag (keys after the query are hidden, by index compare)
-  auto classify = [&](int cidx, uint32_t fl) -> uint32_t {
+  // absent), 8 diag (keys after the query are hidden, by index compare); bits 8..15: key tail of the block (the
+  // block's keys from that one on are hidden from every row: a limit like the end of the keys), 0 for none
+  auto classify = [&](int cidx, uint32_t fl, uint32_t tail) -> uint32_t {
     const int qc0 = cidx * 32, qt0 = (cidx >> 1) * 64, qb = cidx >> 2;
     bool act = (wkb - a.next_blk <= qb) && (qb <= wkb + a.prev_blk) && (wk0 < a.Sk);
     if (causal) act = act && (qt0 + 63 >= wk0);
@@ -721,12 +735,21 @@ ACCT_DEV void fa_bwd_dkdv_body(const FaArgs& a) {
         act = fl != kBlkSkip;                          // class of block (qb, wkb)
         apply_mask = fl == kBlkApply;
         if (fl == kBlkTriu) { diag = true; act = qt0 + 63 >= wk0; }
+        if (apply_mask && tail) {
+          apply_mask = false;
+          act = wk0 < wkb * 128 + (int)tail;            // (else every key of the pair is hidden)
+        } else {
+          tail = 0;
+        }
+      } else {
+        tail = 0;
       }
-    } else if (MASKT && a.mask_kind == kMaskTile) {
-      apply_mask = wkb == qb;
+    } else {
+      tail = 0;
+      if (MASKT && a.mask_kind == kMaskTile) apply_mask = wkb == qb;
     }
-    const bool limits = (diag && (wk0 + WK - 1 > qc0)) || (wk0 + WK > a.Sk) || (qc0 + 32 > a.Sq);
-    return (act ? 1u : 0u) | (apply_mask ? 2u : 0u) | (limits ? 4u : 0u) | (diag ? 8u : 0u);
+    const bool limits = (diag && (wk0 + WK - 1 > qc0)) || (wk0 + WK > a.Sk) || (qc0 + 32 > a.Sq) || (tail && wk0 + WK > wkb * 128 + (int)tail);
+    return (act ? 1u : 0u) | (apply_mask ? 2u : 0u) | (limits ? 4u : 0u) | (diag ? 8u : 0u) | (tail << 8);
   };
 
   if (i_lo <= i_hi) {
@@ -766,14 +789,16 @@ ACCT_DEV void fa_bwd_dkdv_body(const FaArgs& a) {
       for (int t = 0; t < 4; t++) foff4_kept[t] = l32 * C::PITCH + swz_off(2 * t + g, C::swz(l32));
     }
     const uint8_t* flcol = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + (int64_t)mb * a.Tr * a.Tc + wkb : nullptr;
-    if (!flwin_ready) flwin.init_descending(flcol, a.Tc, c_lo >> 2, c_hi >> 2, lane);
+    if (!flwin_ready) flwin.init_descending(flcol, a.Tc, c_lo >> 2, c_hi >> 2, lane, (!BIAS && flcol && a.blktail) ? a.blktail + (flcol - a.blkflags) : nullptr);
     for (int n = 0; n <= npos; n++) {
       if ((n & 1) && (n >> 1) + 1 < ntile) stage(i_hi - ((n >> 1) + 1), smem + ((((n >> 1) + 1) & 1) * STAGEB));
       const int cpos = __builtin_amdgcn_readfirstlane(krole ? n - 1 : n);   // position of the chunk this wave works on in this step (wave-uniform: scalar)
       if (cpos >= 0 && cpos < npos) {
         const int cidx = chunk_at(cpos);
-        const uint32_t cls = classify(cidx, flwin.get(cidx >> 2, lane));
+        const uint32_t fl_cur = flwin.get(cidx >> 2, lane);
+        const uint32_t cls = classify(cidx, fl_cur, (MASKT && !BIAS) ? flwin.tail(cidx >> 2) : 0u);
         const bool act = cls & 1u, apply_mask = cls & 2u, limits = cls & 4u, diag = cls & 8u;
+        const int key_end = (cls >> 8) ? min(a.Sk, wkb * 128 + (int)(cls >> 8)) : a.Sk;   // keys from here on are absent or hidden from every row
         const bool edge = (BIAS && !bias_staged && !row_bias) || apply_mask || limits;   // (a staged or per-key bias is already inside the scores)
         if (act) {
           const int c = cidx & 1, qc0 = cidx * 32;
@@ -901,7 +926,7 @@ ACCT_DEV void fa_bwd_dkdv_body(const FaArgs& a) {
                 const int kv = wk0 + 32 * gk + l32;
                 int lo = diag ? kv - qc0 - 4 * g : -64;         // chunk rows below it come before the key
                 int hi = a.Sq - 1 - qc0 - 4 * g;                // last query row that exists
-                if (kv >= a.Sk) hi = -64;
+                if (kv >= key_end) hi = -64;
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                   const int cr = 8 * (r >> 2) + (r & 3);

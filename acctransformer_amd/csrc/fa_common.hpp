@@ -110,6 +110,8 @@ struct FaArgs {
   float* dkdv_part;                    // q_split > 1: per-slice dK / dV sums of the dK/dV kernel, [q_split][workgroup][wave][regs x 64 lanes]
   const uint8_t* mask; const uint8_t* drop; const void* alibi;   // mask / drop: elements of mask_es / drop_es bytes
   const uint8_t* blkflags;             // [MB, Tr, Tc] block classes of a dense mask
+  const uint8_t* blktail;              // [MB, Tr, Tc] or null: t > 0 for a mixed block whose every row masks exactly the keys from
+                                       // the block's t-th on (key padding: no mask loads there, an index compare); else 0
   const uint32_t* droprow;             // [B*N*Sq, droprow_w] keep bits of the dropout mask by query row: bit k of word w = drop[row][32w+k] != 0
   const uint32_t* dropcol;             // [B*N, Tr, Sk, 4] the same by key column: bit r of the 128-bit entry = drop[128*qb + r][key] != 0
   const uint32_t* colbits;             // [MB, Tr, Sk, 4] dense mask of the 'apply' blocks packed by key column: bit r of the
@@ -170,30 +172,36 @@ ACCT_DEV void trim_dead_tiles(int& lo, int& hi, int lane, F dead) {
 // for lies outside it.
 struct BlkClassWindow {
   const uint8_t* p;
+  const uint8_t* pt = nullptr;        // the same line of the key-tail table (FaArgs::blktail), or null
   int64_t stride;
   int first, last, base;
   uint64_t b0, b1;
-  ACCT_DEV void init(const uint8_t* p_, int64_t stride_, int first_, int last_, int lane) {
-    p = p_; stride = stride_; first = first_; last = last_;
+  uint32_t tl = 0;                    // lane l: key tail of block base + l
+  ACCT_DEV void init(const uint8_t* p_, int64_t stride_, int first_, int last_, int lane, const uint8_t* tails_line = nullptr) {
+    p = p_; pt = tails_line; stride = stride_; first = first_; last = last_;
     load(first, lane);
   }
-  ACCT_DEV void init_descending(const uint8_t* p_, int64_t stride_, int first_, int last_, int lane) {
-    p = p_; stride = stride_; first = first_; last = last_;
+  ACCT_DEV void init_descending(const uint8_t* p_, int64_t stride_, int first_, int last_, int lane, const uint8_t* tails_line = nullptr) {
+    p = p_; pt = tails_line; stride = stride_; first = first_; last = last_;
     load(max(first_, last_ - 63), lane);
   }
   // The window of the blocks [lo, hi] of line `own` and, in the same round trip to memory, the part of [lo, hi]
   // that is not 'skip' in every one of the `n` lines line0 .. line0 + n - 1 (the row or column blocks a
   // workgroup covers; line l, block x sits at tbl[l * line_step + x * stride]): lo and hi shrink to it (lo > hi
   // when nothing is left).  For at most 64 blocks; returns false, with nothing done, when there are more.
-  ACCT_DEV bool init_trimmed(const uint8_t* tbl, int64_t stride_, int64_t line_step, int line0, int n, int own, int& lo, int& hi, int lane) {
+  // `tails`: the key-tail table, indexed like tbl, or null.
+  ACCT_DEV bool init_trimmed(const uint8_t* tbl, int64_t stride_, int64_t line_step, int line0, int n, int own, int& lo, int& hi, int lane,
+                             const uint8_t* tails = nullptr) {
     if (hi - lo >= 64 || n > 2) return false;
     p = tbl + (int64_t)own * line_step; stride = stride_; first = lo; last = hi; base = lo;
+    pt = tails ? tails + (int64_t)own * line_step : nullptr;
     const int blk = lo + lane;
     const bool in = blk <= hi;
     // (all loads are issued before the first ballot waits for one)
     const uint32_t f0 = in ? tbl[(int64_t)line0 * line_step + blk * stride_] : (uint32_t)kBlkSkip;
     const uint32_t f1 = (in && n > 1) ? tbl[(int64_t)(line0 + 1) * line_step + blk * stride_] : (uint32_t)kBlkSkip;
     const uint32_t fo = own == line0 ? f0 : (own == line0 + 1 && n > 1 ? f1 : (in ? p[blk * stride_] : 0u));
+    tl = (pt && in) ? pt[blk * stride_] : 0u;
     const uint64_t live = __ballot(in && !(f0 == kBlkSkip && f1 == kBlkSkip));
     b0 = __ballot(in && (fo & 1u));
     b1 = __ballot(in && (fo & 2u));
@@ -209,6 +217,7 @@ struct BlkClassWindow {
     base = first;
     const int blk = first + lane;
     const uint32_t f = (p && blk <= last) ? p[blk * stride] : 0u;
+    tl = (pt && blk <= last) ? pt[blk * stride] : 0u;
     b0 = __ballot(f & 1u);
     b1 = __ballot(f & 2u);
   }
@@ -218,6 +227,8 @@ struct BlkClassWindow {
     const int sh = blk - base;
     return (uint32_t)((b0 >> sh) & 1u) | ((uint32_t)((b1 >> sh) & 1u) << 1);
   }
+  // key tail of the block that get() was last asked for (0: none)
+  ACCT_DEV uint32_t tail(int blk) { return (uint32_t)__builtin_amdgcn_readlane((int)tl, blk - base); }
 };
 
 // True when the block classes of a dense mask say that, inside the band, the `n` (<= 2) lines line0 .. of the class

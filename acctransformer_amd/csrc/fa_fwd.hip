@@ -64,7 +64,8 @@ ACCT_DEV void fa_fwd_body(const FaArgs& a) {
     // band, one round trip to memory yields both the trimmed range and the wave's class window.
     const uint8_t* fl = a.blkflags + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc;
     int b_lo = j_lo / TPB, b_hi = j_hi / TPB;
-    if (j_lo <= j_hi && flwin.init_trimmed(fl, 1, a.Tc, qb_lo, qb_hi - qb_lo + 1, min(wqb, qb_hi), b_lo, b_hi, lane)) {
+    const uint8_t* tails = a.blktail ? a.blktail + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc : nullptr;
+    if (j_lo <= j_hi && flwin.init_trimmed(fl, 1, a.Tc, qb_lo, qb_hi - qb_lo + 1, min(wqb, qb_hi), b_lo, b_hi, lane, tails)) {
       j_lo = max(j_lo, b_lo * TPB);
       j_hi = min(j_hi, b_hi * TPB + TPB - 1);
       flwin_ready = true;
@@ -165,8 +166,9 @@ ACCT_DEV void fa_fwd_body(const FaArgs& a) {
   ACCT_LDS char* drop_lds = smem + 4 * TILEB + NW * BIASB + wave * (2 * DropStage::BYTES);
   // ---- the phases of a tile step: classification, S^T = K Q^T, online softmax, O^T += V^T P^T ----
   const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
-  if (!flwin_ready && j_lo <= j_hi) flwin.init(flrow, 1, j_lo / TPB, j_hi / TPB, lane);
-  enum : uint32_t { kAct = 1u, kApply = 2u, kDiag = 4u };
+  if (!flwin_ready && j_lo <= j_hi)
+    flwin.init(flrow, 1, j_lo / TPB, j_hi / TPB, lane, (flrow && a.blktail) ? a.blktail + (flrow - a.blkflags) : nullptr);
+  enum : uint32_t { kAct = 1u, kApply = 2u, kDiag = 4u, kTailShift = 8u };   // bits 8..15: key tail of the tile's block (0: none)
   // what this wave does with tile j (tiles must be asked for in ascending order)
   auto classify = [&](int j) -> uint32_t {
     const uint32_t fl_cur = flwin.get(j / TPB, lane);
@@ -176,14 +178,20 @@ ACCT_DEV void fa_fwd_body(const FaArgs& a) {
     act = act && (kv0 < wkv_limit);
     bool apply_mask = false;
     bool diag = causal;                                     // keys after the query are hidden, by index compare
+    uint32_t tail = 0;
     if (MASKT && a.mask_kind == kMaskDense && act) {
       act = fl_cur != kBlkSkip;
       apply_mask = fl_cur == kBlkApply;
       if (fl_cur == kBlkTriu) { diag = true; act = kv0 <= wq_end - 1; }
+      if (apply_mask && (tail = flwin.tail(kvb)) != 0) {
+        // every row of the block hides exactly the keys from its tail-th on: an index compare, no mask loads
+        apply_mask = false;
+        act = kv0 < kvb * 128 + (int)tail;
+      }
     } else if (MASKT && a.mask_kind == kMaskTile) {
       apply_mask = wqb == kvb;
     }
-    return (act ? kAct : 0u) | (apply_mask ? kApply : 0u) | (diag ? kDiag : 0u);
+    return (act ? kAct : 0u) | (apply_mask ? kApply : 0u) | (diag ? kDiag : 0u) | (tail << kTailShift);
   };
   // stage key rows [j BN, (j+1) BN) of K or V into an LDS tile
   auto stage_tile = [&](const TileDma<T, D, BN, NW>& dma, const T* base, int64_t ss, int j, ACCT_LDS char* dst) {
@@ -258,8 +266,10 @@ ACCT_DEV void fa_fwd_body(const FaArgs& a) {
   auto softmax = [&](int j, int buf, uint32_t info, f32x16 (&s)[QG][KT], V8 (&pf)[QG][KT][2]) {
     const int kv0 = j * BN;
     const bool apply_mask = MASKT && (info & kApply), diag = info & kDiag;
+    const int tail = MASKT ? (int)((info >> kTailShift) & 0xffu) : 0;
+    const int last_key = tail ? min(a.Sk, (j / TPB) * 128 + tail) - 1 : a.Sk - 1;     // last key that exists and is not behind a key tail
     // element (gq, c, r): q = wq0 + 32 gq + l32 ; kv = kv0 + 32 c + 8 (r/4) + 4 g + r%4
-    const bool edge = apply_mask || (diag && (kv0 + BN - 1 > wq0)) || (kv0 + BN > a.Sk);
+    const bool edge = apply_mask || (diag && (kv0 + BN - 1 > wq0)) || (kv0 + BN - 1 > last_key);
 #pragma unroll
     for (int gq = 0; gq < QG; gq++) {
       const int qrow = wq0 + 32 * gq + l32;
@@ -317,7 +327,7 @@ ACCT_DEV void fa_fwd_body(const FaArgs& a) {
           // Keys after the query (causal diagonal) and keys past Sk are removed outright: with the additive
           // mask their probability underflows to exactly 0 as well (the diagonal key is always visible), so
           // the result is the same bit for bit at a third of the vector instructions.
-          int vis = a.Sk - 1 - kv0 - 4 * g;                  // last visible key, relative to this lane's first
+          int vis = last_key - kv0 - 4 * g;                  // last visible key, relative to this lane's first
           if (diag) vis = min(vis, qrow - kv0 - 4 * g);
           // (compare and select through VCC: see select_if_gt)
           const float ninf = -INFINITY;

@@ -39,6 +39,8 @@ bool launch_variants_complete();
 
 // classify the 128x128 blocks of a dense mask into clean / apply / skip / causal diagonal and, with `colbits`
 // non-null, pack its 'apply' blocks into per-key-column bitmaps [MB, Tr, Sk, 4 x u32] (one launch for aligned masks)
+// true when launch_mask_blocks takes its one-launch path, which also fills the key-tail table behind the classes
+bool mask_prepass_is_fused(const FaArgs& a);
 hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, uint32_t* colbits, int MB, hipStream_t st);
 // pack the dropout mask into keep bits by query row [B*N, Sq, droprow_w] and / or by key column [B*N, Tr, Sk, 4]
 hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st);

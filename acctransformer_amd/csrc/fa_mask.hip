@@ -32,16 +32,17 @@ constexpr uint8_t kBlkAllMasked = 255;  // provisional: resolved to skip or appl
 // visible) and for key padding (the first keys are); where it fails although the rows do see keys elsewhere,
 // the block is classed 'apply' instead of 'skip', which gives the same results bit for bit, only slower.
 template <int ES>
-__global__ void __launch_bounds__(256) fa_mask_prepass_kernel(const FaArgs a, uint8_t* flags, uint32_t* colbits) {
+__global__ void __launch_bounds__(256) fa_mask_prepass_kernel(const FaArgs a, uint8_t* flags, uint8_t* tails, uint32_t* colbits) {
   __shared__ unsigned long long s_bits[128][2];         // nonzero bits of the block: [row][column half]
   __shared__ unsigned long long s_seen[2];              // rows (bit = row % 64) with an unmasked key in the blocks probed
+  __shared__ int s_lead[2];                             // unmasked leading columns of the block's first row, per column half
   const int kvb = blockIdx.x % a.Tc, qb = (blockIdx.x / a.Tc) % a.Tr, mb = blockIdx.x / (a.Tc * a.Tr);
   const int tid = threadIdx.x;
   int lo = max(0, qb - a.prev_blk), hi = min(a.Tc - 1, qb + a.next_blk);
   if (a.row_prefix) hi = min(hi, ((qb * 128 / a.row_prefix + 1) * a.row_prefix - 1) / 128);
   const int64_t blk = ((int64_t)mb * a.Tr + qb) * a.Tc + kvb;
   if (kvb < lo || kvb > hi) {                           // outside the band: never visited
-    if (tid == 0) flags[blk] = kBlkClean;
+    if (tid == 0) { flags[blk] = kBlkClean; tails[blk] = 0; }
     return;
   }
   const int rib = tid & 127, half = tid >> 7, row = qb * 128 + rib, c0 = half * 64;
@@ -106,7 +107,20 @@ __global__ void __launch_bounds__(256) fa_mask_prepass_kernel(const FaArgs a, ui
     }
     if (!ok) cls = kBlkApply;
   }
-  if (tid == 0) flags[blk] = cls;
+  // A mixed block in which every row masks exactly the columns from the t-th on (1 <= t <= 127; key padding that
+  // ends inside the block): the forward and dQ kernels compare key indices with t there instead of loading mask
+  // bytes.  t is taken from the block's first row (which always exists) and checked against every row.
+  int tail = 0;
+  if (cls == kBlkApply) {                               // (uniform)
+    if (rib == 0) s_lead[half] = nz ? __builtin_ctzll(nz) : 64;
+    __syncthreads();
+    const int t = s_lead[0] < 64 ? s_lead[0] : 64 + s_lead[1];
+    const int rel = t - c0;                             // this thread's columns from bit `rel` on are masked
+    const unsigned long long want = rel <= 0 ? ~0ull : (rel >= 64 ? 0ull : (~0ull << rel));
+    const int differs = __syncthreads_or(row < a.Sq && ((nz ^ want) & valid) != 0);
+    if (!differs && t >= 1 && t <= 127) tail = t;
+  }
+  if (tid == 0) { flags[blk] = cls; tails[blk] = (uint8_t)tail; }
   if (cls == kBlkApply && colbits) {
     // the block packed by key column: 128 bits per key, bit r = mask[128 qb + r][key]
     s_bits[rib][half] = nz;
@@ -382,7 +396,7 @@ hipError_t launch_drop_bits(const FaArgs& a, uint32_t* rowbits, uint32_t* colbit
 }
 
 // true when launch_mask_blocks takes the fast path, which also writes the column bitmaps
-static bool mask_prepass_is_fused(const FaArgs& a) {
+bool mask_prepass_is_fused(const FaArgs& a) {
   // every 16-element piece of a row is 16-byte aligned and entirely inside or outside the row
   return (((uintptr_t)a.mask | (uintptr_t)a.Sk | (uintptr_t)a.mask_sb) & 15) == 0;
 }
@@ -390,8 +404,9 @@ static bool mask_prepass_is_fused(const FaArgs& a) {
 hipError_t launch_mask_blocks(const FaArgs& a, uint8_t* flags, uint32_t* colbits, int MB, hipStream_t st) {
   if (mask_prepass_is_fused(a)) {
     const dim3 grid((unsigned)((long long)MB * a.Tr * a.Tc));
-    if (a.mask_es == 2) hipLaunchKernelGGL(fa_mask_prepass_kernel<2>, grid, dim3(256), 0, st, a, flags, colbits);
-    else hipLaunchKernelGGL(fa_mask_prepass_kernel<1>, grid, dim3(256), 0, st, a, flags, colbits);
+    uint8_t* tails = flags + (size_t)MB * a.Tr * a.Tc;  // (the key-tail table follows the classes)
+    if (a.mask_es == 2) hipLaunchKernelGGL(fa_mask_prepass_kernel<2>, grid, dim3(256), 0, st, a, flags, tails, colbits);
+    else hipLaunchKernelGGL(fa_mask_prepass_kernel<1>, grid, dim3(256), 0, st, a, flags, tails, colbits);
     return hipGetLastError();
   }
   const dim3 grid((unsigned)(MB * a.Tr));
