@@ -235,6 +235,35 @@ def test_padding_mask_with_dropout():
                                       drop_mask=drop, keep_prob=0.9))
 
 
+@pytest.mark.parametrize("side", ["none", "dropout", "full_bias", "row_bias_dropout", "causal_too"])
+@pytest.mark.parametrize("Sq, Sk, lens", [(512, 512, (1, 127, 129, 300)), (384, 640, (64, 192, 513, 640)), (256, 400, (128, 399, 257, 16))])
+def test_key_padding_that_ends_inside_a_block(Sq, Sk, lens, side):
+    # per-sequence key padding whose boundary falls in the first, a middle or the last (here also partial) 128-key
+    # block, at a block edge, or on the edge of a 64-key tile: the boundary block of every row block is mixed, with the
+    # same key tail in every row; with a causal mask on top the diagonal blocks are mixed without a common tail
+    B, N, D = len(lens), 2, 128
+    q, dO = (_gen((B, N, Sq, D), s) for s in (401, 404))
+    k, v = (_gen((B, N, Sk, D), s) for s in (402, 403))
+    m = np.ascontiguousarray(np.broadcast_to(np.arange(Sk)[None, None, :] >= np.asarray(lens)[:, None, None], (B, Sq, Sk)), dtype=np.uint8)
+    if side == "causal_too":
+        m = np.maximum(m, np.triu(np.ones((1, Sq, Sk), np.uint8), 1))
+    scale = D ** -0.5
+    kw, okw = dict(scale=scale, mask_kind=_capi.MASK_DENSE_U8, attn_mask=m), dict(scale=scale, attn_mask=m)
+    if "dropout" in side:
+        kw.update(keep_prob=0.8, drop_seed=5 << 20, drop_offset=3)
+        okw.update(drop_mask=phx.dropout_keep_mask(B, N, Sq, Sk, 5 << 20, 3, 0.8), keep_prob=phx.keep_threshold(0.8) / 256.0)
+        v = (0.5 * v.float()).half()                     # (rows with one visible key: see test_dense_causal_forms)
+    if "bias" in side:
+        al = (0.3 * torch.randn((1, N, Sq, Sk) if side == "full_bias" else (1, N, 1, Sk), generator=torch.Generator().manual_seed(9))).half()
+        kw.update(alibi=al); okw.update(alibi=al.float().numpy())
+    _check_all(q, k, v, dO, okw, _run(q, k, v, dO, **kw), saved_o=True)
+    # the same mask in the reference's 2-byte form gives the same bits
+    res8 = _run(q, k, v, dO, **kw)
+    kw.update(mask_kind=_capi.MASK_DENSE_F16, attn_mask=torch.from_numpy(m).half())
+    res16 = _run(q, k, v, dO, **kw)
+    assert torch.equal(res8[0], res16[0]) and all(torch.equal(a, b) for a, b in zip(res8[2], res16[2]))
+
+
 @pytest.mark.parametrize("Sq, Sk", [(300, 333), (1100, 1100), (130, 2050)])
 def test_ragged_dropout_with_random_mask(Sq, Sk):
     # lengths off every vector width and tile edge: the keep-bit packing (16-byte loads, 1024-key spans,
