@@ -79,7 +79,7 @@ ACCT_DEV void fa_bwd_dq_body(const FaArgs& a) {
     int b_lo = j_lo >> 1, b_hi = j_hi >> 1;
     // (the dropout variants have no register to spare for the key tails -- one more spill costs them 5 % on every
     // tile -- and read such blocks as mask bytes)
-    const uint8_t* tails = (!DROP && a.blktail) ? a.blktail + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc : nullptr;
+    const uint8_t* tails = a.blktail ? a.blktail + ((int64_t)(a.mask_sb ? b : 0) * a.Tr) * a.Tc : nullptr;
     if (j_lo <= j_hi && flwin.init_trimmed(fl, 1, a.Tc, qb_lo, qb_hi - qb_lo + 1, min(wqb, qb_hi), b_lo, b_hi, lane, tails)) {
       j_lo = max(j_lo, b_lo * 2);
       j_hi = min(j_hi, b_hi * 2 + 1);
@@ -188,7 +188,7 @@ ACCT_DEV void fa_bwd_dq_body(const FaArgs& a) {
 
     // block classes of a dense mask: 64 blocks at a time into scalar registers
     const uint8_t* flrow = (MASKT && a.mask_kind == kMaskDense) ? a.blkflags + ((int64_t)mb * a.Tr + wqb) * a.Tc : nullptr;
-    if (!flwin_ready) flwin.init(flrow, 1, j_lo >> 1, j_hi >> 1, lane, (!DROP && flrow && a.blktail) ? a.blktail + (flrow - a.blkflags) : nullptr);
+    if (!flwin_ready) flwin.init(flrow, 1, j_lo >> 1, j_hi >> 1, lane, (flrow && a.blktail) ? a.blktail + (flrow - a.blkflags) : nullptr);
     for (int j = j_lo; j <= j_hi; j++) {
       const uint32_t fl_cur = flwin.get(j >> 1, lane);
       const int buf = (j - j_lo) & 1;
@@ -217,7 +217,7 @@ ACCT_DEV void fa_bwd_dq_body(const FaArgs& a) {
         act = fl_cur != kBlkSkip;
         apply_mask = fl_cur == kBlkApply;
         if (fl_cur == kBlkTriu) { diag = true; act = kv0 <= wq_end - 1; }
-        if (apply_mask && !DROP) {
+        if (apply_mask) {
           const int tail = (int)flwin.tail(kvb);
           if (tail) {
             // every row of the block hides exactly the keys from its tail-th on: an index compare, no mask loads

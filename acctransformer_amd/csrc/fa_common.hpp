@@ -176,7 +176,8 @@ struct BlkClassWindow {
   int64_t stride;
   int first, last, base;
   uint64_t b0, b1;
-  uint32_t tl = 0;                    // lane l: key tail of block base + l
+  int tail_blk = -1;                  // the first block of the window with a key tail, and that tail (scalar registers; further
+  uint32_t tail_t = 0;                // such blocks of the window are read as mixed blocks: same results)
   ACCT_DEV void init(const uint8_t* p_, int64_t stride_, int first_, int last_, int lane, const uint8_t* tails_line = nullptr) {
     p = p_; pt = tails_line; stride = stride_; first = first_; last = last_;
     load(first, lane);
@@ -201,7 +202,7 @@ struct BlkClassWindow {
     const uint32_t f0 = in ? tbl[(int64_t)line0 * line_step + blk * stride_] : (uint32_t)kBlkSkip;
     const uint32_t f1 = (in && n > 1) ? tbl[(int64_t)(line0 + 1) * line_step + blk * stride_] : (uint32_t)kBlkSkip;
     const uint32_t fo = own == line0 ? f0 : (own == line0 + 1 && n > 1 ? f1 : (in ? p[blk * stride_] : 0u));
-    tl = (pt && in) ? pt[blk * stride_] : 0u;
+    note_tail((pt && in) ? pt[blk * stride_] : 0u);
     const uint64_t live = __ballot(in && !(f0 == kBlkSkip && f1 == kBlkSkip));
     b0 = __ballot(in && (fo & 1u));
     b1 = __ballot(in && (fo & 2u));
@@ -217,7 +218,7 @@ struct BlkClassWindow {
     base = first;
     const int blk = first + lane;
     const uint32_t f = (p && blk <= last) ? p[blk * stride] : 0u;
-    tl = (pt && blk <= last) ? pt[blk * stride] : 0u;
+    note_tail((pt && blk <= last) ? pt[blk * stride] : 0u);
     b0 = __ballot(f & 1u);
     b1 = __ballot(f & 2u);
   }
@@ -227,8 +228,18 @@ struct BlkClassWindow {
     const int sh = blk - base;
     return (uint32_t)((b0 >> sh) & 1u) | ((uint32_t)((b1 >> sh) & 1u) << 1);
   }
-  // key tail of the block that get() was last asked for (0: none)
-  ACCT_DEV uint32_t tail(int blk) { return (uint32_t)__builtin_amdgcn_readlane((int)tl, blk - base); }
+  // tl: lane l holds the key tail of block base + l
+  ACCT_DEV void note_tail(uint32_t tl) {
+    const uint64_t any = __ballot(tl != 0);
+    tail_blk = -1; tail_t = 0;
+    if (any) {
+      const int l = __builtin_ctzll(any);
+      tail_blk = base + l;
+      tail_t = (uint32_t)__builtin_amdgcn_readlane((int)tl, l);
+    }
+  }
+  // key tail of a block inside the window (0: none, or not the window's first)
+  ACCT_DEV uint32_t tail(int blk) const { return blk == tail_blk ? tail_t : 0u; }
 };
 
 // True when the block classes of a dense mask say that, inside the band, the `n` (<= 2) lines line0 .. of the class
