@@ -234,15 +234,16 @@ hipError_t launch_mask_colbits(const FaArgs& a, const uint8_t* flags, uint32_t* 
 // Column entries of the dropout bitmaps, written whole.  The four waves of a workgroup each hold, per lane and for
 // sixteen keys, the 32-bit word of their 32 rows; a key's 16-byte entry is the four waves' words.  Written straight
 // from the waves every entry would be four 4-byte stores from four places; instead the words cross LDS and every
-// thread stores complete entries, consecutive threads consecutive entries.  key_of(lane, e): the key of a lane's
-// e-th word.  (One spare entry after every sixteen keeps the word stores of a wave on different banks.)
+// thread stores complete entries, consecutive threads consecutive entries.  cw[e]: bit r = row r of the wave's 32;
+// key_of(lane, e): the key of a lane's e-th word.  (One spare entry after every sixteen keeps the word stores of a
+// wave on different banks.)
 template <typename KeyOf>
 ACCT_DEV void store_col_entries(uint32_t* s_cw, const uint32_t (&cw)[16], int wave, int lane, int key0, int Sk, uint32_t* out,
                                 KeyOf key_of) {
 #pragma unroll
   for (int e = 0; e < 16; e++) {
     const int k = key_of(lane, e);                       // 0 .. 1023 within the span
-    s_cw[(k + (k >> 4)) * 4 + wave] = __builtin_bitreverse32(cw[e]);
+    s_cw[(k + (k >> 4)) * 4 + wave] = cw[e];
   }
   __syncthreads();
 #pragma unroll
@@ -292,46 +293,70 @@ __global__ void __launch_bounds__(256) fa_drop_bits_kernel(const FaArgs a, uint3
   const bool writer = rowbits && lane % LPW == 0;
   uint32_t* rowout = rowbits + ((int64_t)bh * a.Sq + qb * 128 + 32 * i) * a.droprow_w + widx;
   const int nrow = min(128, a.Sq - qb * 128);
-  uint32_t cw[16];                                      // per key: the word of these 32 rows, most significant bit first
+  // cw[j]: the keep bits (bit e = this lane's key e) of rows j (low half) and j + 16 (high half) of the wave's 32
+  uint32_t cw[16];
 #pragma unroll
   for (int e = 0; e < 16; e++) cw[e] = 0u;
-#pragma unroll 16
-  for (int r = 0; r < 32; r++) {
-    const int rr = 32 * i + r;
-    uint32_t nz = 0;                                    // bit KH*h + e: key e of this lane's load h is kept
+  for (int rh = 0; rh < 2; rh++) {
 #pragma unroll
-    for (int h = 0; h < NH; h++) {
-      if (rr < nrow && !dead[h]) {
-        if (vec[h]) {
-          const u32x4 v = *reinterpret_cast<const u32x4*>(p[h]);
+    for (int j = 0; j < 16; j++) {
+      const int rr = 32 * i + 16 * rh + j;
+      uint32_t nz = 0;                                  // bit KH*h + e: key e of this lane's load h is kept
 #pragma unroll
-          for (int w = 0; w < 4; w++) {
-            if (ES == 1) {
+      for (int h = 0; h < NH; h++) {
+        if (rr < nrow && !dead[h]) {
+          if (vec[h]) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(p[h]);
 #pragma unroll
-              for (int e = 0; e < 4; e++) nz |= (((v[w] >> (8 * e)) & 0xffu) != 0 ? 1u : 0u) << (4 * w + e);
-            } else {
-              nz |= (((v[w] & 0x7fffu) != 0 ? 1u : 0u) | (((v[w] >> 16) & 0x7fffu) != 0 ? 2u : 0u)) << (KH * h + 2 * w);
+            for (int w = 0; w < 4; w++) {
+              if (ES == 1) {
+                // bit 8e: byte e is nonzero (no carry leaves a byte); then the four bits side by side
+                const uint32_t y = ((((v[w] & 0x7f7f7f7fu) + 0x7f7f7f7fu) | v[w]) >> 7) & 0x01010101u;
+                nz |= ((y | (y >> 7) | (y >> 14) | (y >> 21)) & 0xfu) << (4 * w);
+              } else {
+                // 2-byte floating-point elements: nonzero apart from the sign bit
+                const uint32_t m = v[w] & 0x7fff7fffu;
+                const uint32_t y = (((m + 0x7fff7fffu) | m) >> 15) & 0x00010001u;
+                nz |= ((y | (y >> 15)) & 3u) << (KH * h + 2 * w);
+              }
             }
+          } else {
+            const uint8_t* q = a.drop + ((int64_t)bh * a.Sq + qb * 128 + rr) * a.Sk * ES;
+#pragma unroll
+            for (int e = 0; e < KH; e++)
+              if (kv[h] + e < a.Sk && elem_nonzero<ES>(q, kv[h] + e)) nz |= 1u << (KH * h + e);
           }
-        } else {
-          const uint8_t* q = a.drop + ((int64_t)bh * a.Sq + qb * 128 + rr) * a.Sk * ES;
-#pragma unroll
-          for (int e = 0; e < KH; e++)
-            if (kv[h] + e < a.Sk && elem_nonzero<ES>(q, kv[h] + e)) nz |= 1u << (KH * h + e);
         }
+        p[h] += (int64_t)a.Sk * ES;                     // per-lane pointers walk down the rows
       }
-      p[h] += (int64_t)a.Sk * ES;                       // per-lane pointers walk down the rows
-    }
+      cw[j] |= nz << (16 * rh);
 #pragma unroll
-    for (int e = 0; e < 16; e++) cw[e] = (cw[e] << 1) | ((nz >> e) & 1u);
-#pragma unroll
-    for (int h = 0; h < NH; h++) {
-      uint32_t x = ((nz >> (KH * h)) & ((1u << KH) - 1u)) << (KH * (lane % LPW));
-      x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xf, 0xf, true);                   // lane ^ 1
-      if (LPW == 4) x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xf, 0xf, true);     // lane ^ 2
-      if (writer && rr < nrow && widx + 16 * h < a.droprow_w) rowout[16 * h] = x;
+      for (int h = 0; h < NH; h++) {
+        uint32_t x = ((nz >> (KH * h)) & ((1u << KH) - 1u)) << (KH * (lane % LPW));
+        x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xf, 0xf, true);                   // lane ^ 1
+        if (LPW == 4) x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xf, 0xf, true);     // lane ^ 2
+        if (writer && rr < nrow && widx + 16 * h < a.droprow_w) rowout[16 * h] = x;
+      }
+      rowout += a.droprow_w;
     }
-    rowout += a.droprow_w;
+  }
+  // The column words are the transpose of that 32 x 16 bit matrix: two 16 x 16 transposes side by side in the
+  // sixteen registers (sub-blocks of 8, 4, 2, 1 swapped across the diagonal), after which bit r of cw[e] is the
+  // keep bit of row r and key e.  (Shifting every key's bit into sixteen words row by row cost five times as many
+  // instructions; this pass is bound by them, not by memory, once lanes of hidden key blocks load nothing.)
+  {
+    uint32_t mask = 0x00ff00ffu;
+#pragma unroll
+    for (int sft = 8; sft >= 1; sft >>= 1) {
+#pragma unroll
+      for (int k = 0; k < 16; k++) {
+        if (k & sft) continue;
+        const uint32_t t = ((cw[k] >> sft) ^ cw[k + sft]) & mask;
+        cw[k + sft] ^= t;
+        cw[k] ^= t << sft;
+      }
+      mask ^= mask << (sft >> 1);
+    }
   }
   if (colbits)
     store_col_entries(s_cw, cw, i, lane, span * 1024, a.Sk, colbits + ((int64_t)bh * a.Tr + qb) * a.Sk * 4,
@@ -377,9 +402,12 @@ __global__ void __launch_bounds__(256) fa_drop_philox_kernel(const FaArgs a, uin
       rowout += a.droprow_w;
     }
   }
-  if (colbits)
+  if (colbits) {
+#pragma unroll
+    for (int t = 0; t < 16; t++) cw[t] = __builtin_bitreverse32(cw[t]);
     store_col_entries(s_cw, cw, i, lane, span * 1024, a.Sk, colbits + ((int64_t)bh * a.Tr + qb) * a.Sk * 4,
                       [](int l, int t) { return 32 * (l >> 1) + 8 * (t >> 2) + 4 * (l & 1) + (t & 3); });
+  }
 }
 
 hipError_t launch_drop_philox(const FaArgs& a, uint32_t* rowbits, uint32_t* colbits, hipStream_t st) {
