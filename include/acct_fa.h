@@ -130,7 +130,9 @@ typedef struct acct_fa_params {
   /* What the pre-passes derive from attn_mask, shared between the calls of one training step (fields added in
      version 108; no counterpart in the reference, whose kernels read the mask tile by tile,
      T/attention.py:357-371).  A dense mask is classified block by block (clean / apply / skip / causal
-     diagonal) and, for the dK/dV kernel, packed by key column; the compact tile is packed by key column.
+     diagonal; for a block in which every row hides exactly the keys from one position on -- key padding that
+     ends inside the block -- that position) and, for the dK/dV kernel, packed by key column; the compact tile
+     is packed by key column.
      With mask_bits == NULL every call runs the pre-passes into its own workspace.  With mask_bits pointing
      at acct_fa_mask_bits_bytes(p) bytes of device memory (256-byte aligned) that the caller keeps across the
      calls, a call with mask_bits_filled == 0 runs them into that buffer and a call with
