@@ -616,7 +616,7 @@ ACCT_DEV void fa_bwd_dkdv_body(const FaArgs& a) {
     i_hi = min(i_hi, (slice + 1) * per - 1);
   }
   const int wkb = wk0 / 128;
-  BlkClassWindow flwin;                               // block classes of a dense mask: 64 blocks at a time in scalar registers
+  BlkClassWindowLaneTails flwin;                      // block classes of a dense mask: 64 blocks at a time in scalar registers
   bool flwin_ready = false;
   if (MASKT && a.mask_kind == kMaskDense) {
     // query tiles at either end whose blocks are wholly masked for every key block of this workgroup are
@@ -750,7 +750,7 @@ ACCT_DEV void fa_bwd_dkdv_body(const FaArgs& a) {
       tail = 0;
       if (MASKT && a.mask_kind == kMaskTile) apply_mask = wkb == qb;
     }
-    const bool limits = (diag && (wk0 + WK - 1 > qc0)) || (wk0 + WK > a.Sk) || (qc0 + 32 > a.Sq) || (tail && wk0 + WK > wkb * 128 + (int)tail);
+    const bool limits = (diag && (wk0 + WK - 1 > qc0)) || (wk0 + WK > a.Sk) || (qc0 + 32 > a.Sq);
     return (act ? 1u : 0u) | (apply_mask ? 2u : 0u) | (limits ? 4u : 0u) | (diag ? 8u : 0u) | (tail << 8);
   };
 
@@ -800,7 +800,10 @@ ACCT_DEV void fa_bwd_dkdv_body(const FaArgs& a) {
         const uint32_t fl_cur = flwin.get(cidx >> 2, lane);
         const uint32_t cls = classify(cidx, fl_cur, (MASKT && !BIAS) ? flwin.tail(cidx >> 2) : 0u);
         const bool act = cls & 1u, apply_mask = cls & 2u, limits = cls & 4u, diag = cls & 8u;
-        const int key_end = (cls >> 8) ? min(a.Sk, wkb * 128 + (int)(cls >> 8)) : a.Sk;   // keys from here on are absent or hidden from every row
+        // keys from key_end on are hidden from every row of the chunk (a key tail): a lane owns a key, so its whole
+        // column of P is zeroed after the probabilities are packed (one AND per packed word)
+        const int key_end = (cls >> 8) ? wkb * 128 + (int)(cls >> 8) : 0x7fffffff;
+        const bool ktail = wk0 + WK > key_end;
         const bool edge = (BIAS && !bias_staged && !row_bias) || apply_mask || limits;   // (a staged or per-key bias is already inside the scores)
         if (act) {
           const int c = cidx & 1, qc0 = cidx * 32;
@@ -928,7 +931,7 @@ ACCT_DEV void fa_bwd_dkdv_body(const FaArgs& a) {
                 const int kv = wk0 + 32 * gk + l32;
                 int lo = diag ? kv - qc0 - 4 * g : -64;         // chunk rows below it come before the key
                 int hi = a.Sq - 1 - qc0 - 4 * g;                // last query row that exists
-                if (kv >= key_end) hi = -64;
+                if (kv >= a.Sk) hi = -64;
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                   const int cr = 8 * (r >> 2) + (r & 3);
@@ -953,9 +956,18 @@ ACCT_DEV void fa_bwd_dkdv_body(const FaArgs& a) {
                     if (DROP) pd[4 * r4 + e] = __uint_as_float(__float_as_uint(p[4 * r4 + e]) & (uint32_t)__builtin_amdgcn_sbfe((int)dcw[gk], 16 * hh + 8 * r4 + e, 1));
                   }
                 }
-                bfr[gk][hh] = pack8<T>(pd);
-                // un-dropped P for the partner, always fp16 (P <= 1: finer than bf16)
-                *reinterpret_cast<ACCT_LDS f16x8*>(px + (2 * gk + hh) * 1024) = pack8<f16>(p);
+                V8 pv = pack8<T>(pd);
+                f16x8 ph = pack8<f16>(p);                  // un-dropped P for the partner, always fp16 (P <= 1: finer than bf16)
+                if (ktail) {
+                  const uint32_t km = wk0 + 32 * gk + l32 < key_end ? 0xffffffffu : 0u;
+                  u32x4 w0 = __builtin_bit_cast(u32x4, pv), w1 = __builtin_bit_cast(u32x4, ph);
+#pragma unroll
+                  for (int e = 0; e < 4; e++) { w0[e] &= km; w1[e] &= km; }
+                  pv = __builtin_bit_cast(V8, w0);
+                  ph = __builtin_bit_cast(f16x8, w1);
+                }
+                bfr[gk][hh] = pv;
+                *reinterpret_cast<ACCT_LDS f16x8*>(px + (2 * gk + hh) * 1024) = ph;
               }
             }
           } else {

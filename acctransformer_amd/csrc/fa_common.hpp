@@ -242,6 +242,70 @@ struct BlkClassWindow {
   ACCT_DEV uint32_t tail(int blk) const { return blk == tail_blk ? tail_t : 0u; }
 };
 
+// The same window with the key tail of EVERY block of the window, in one vector register.  A window along the key
+// axis of a padded batch (forward, dQ) holds one key-tail block, which the two scalar registers above cover; a
+// window along the query axis (the dK/dV kernel's) holds one per query block.
+struct BlkClassWindowLaneTails {
+  const uint8_t* p;
+  const uint8_t* pt = nullptr;        // the same line of the key-tail table (FaArgs::blktail), or null
+  int64_t stride;
+  int first, last, base;
+  uint64_t b0, b1;
+  uint32_t tail_l = 0;                // lane l: key tail of block base + l
+  ACCT_DEV void init(const uint8_t* p_, int64_t stride_, int first_, int last_, int lane, const uint8_t* tails_line = nullptr) {
+    p = p_; pt = tails_line; stride = stride_; first = first_; last = last_;
+    load(first, lane);
+  }
+  ACCT_DEV void init_descending(const uint8_t* p_, int64_t stride_, int first_, int last_, int lane, const uint8_t* tails_line = nullptr) {
+    p = p_; pt = tails_line; stride = stride_; first = first_; last = last_;
+    load(max(first_, last_ - 63), lane);
+  }
+  // The window of the blocks [lo, hi] of line `own` and, in the same round trip to memory, the part of [lo, hi]
+  // that is not 'skip' in every one of the `n` lines line0 .. line0 + n - 1 (the row or column blocks a
+  // workgroup covers; line l, block x sits at tbl[l * line_step + x * stride]): lo and hi shrink to it (lo > hi
+  // when nothing is left).  For at most 64 blocks; returns false, with nothing done, when there are more.
+  // `tails`: the key-tail table, indexed like tbl, or null.
+  ACCT_DEV bool init_trimmed(const uint8_t* tbl, int64_t stride_, int64_t line_step, int line0, int n, int own, int& lo, int& hi, int lane,
+                             const uint8_t* tails = nullptr) {
+    if (hi - lo >= 64 || n > 2) return false;
+    p = tbl + (int64_t)own * line_step; stride = stride_; first = lo; last = hi; base = lo;
+    pt = tails ? tails + (int64_t)own * line_step : nullptr;
+    const int blk = lo + lane;
+    const bool in = blk <= hi;
+    // (all loads are issued before the first ballot waits for one)
+    const uint32_t f0 = in ? tbl[(int64_t)line0 * line_step + blk * stride_] : (uint32_t)kBlkSkip;
+    const uint32_t f1 = (in && n > 1) ? tbl[(int64_t)(line0 + 1) * line_step + blk * stride_] : (uint32_t)kBlkSkip;
+    const uint32_t fo = own == line0 ? f0 : (own == line0 + 1 && n > 1 ? f1 : (in ? p[blk * stride_] : 0u));
+    note_tail((pt && in) ? pt[blk * stride_] : 0u);
+    const uint64_t live = __ballot(in && !(f0 == kBlkSkip && f1 == kBlkSkip));
+    b0 = __ballot(in && (fo & 1u));
+    b1 = __ballot(in && (fo & 2u));
+    if (live) {
+      hi = lo + 63 - __builtin_clzll(live);
+      lo += __builtin_ctzll(live);
+    } else {
+      hi = lo - 1;
+    }
+    return true;
+  }
+  ACCT_DEV void load(int first, int lane) {
+    base = first;
+    const int blk = first + lane;
+    const uint32_t f = (p && blk <= last) ? p[blk * stride] : 0u;
+    note_tail((pt && blk <= last) ? pt[blk * stride] : 0u);
+    b0 = __ballot(f & 1u);
+    b1 = __ballot(f & 2u);
+  }
+  ACCT_DEV uint32_t get(int blk, int lane) {
+    if (blk - base >= 64) load(blk, lane);
+    else if (blk < base) load(max(first, blk - 63), lane);
+    const int sh = blk - base;
+    return (uint32_t)((b0 >> sh) & 1u) | ((uint32_t)((b1 >> sh) & 1u) << 1);
+  }
+  ACCT_DEV void note_tail(uint32_t tl) { tail_l = tl; }
+  ACCT_DEV uint32_t tail(int blk) const { return (uint32_t)__builtin_amdgcn_readlane((int)tail_l, blk - base); }
+};
+
 // True when the block classes of a dense mask say that, inside the band, the `n` (<= 2) lines line0 .. of the class
 // table that a workgroup covers hold exactly the causal pattern: clean before the diagonal, the causal diagonal
 // class on it, skipped after it.  Such a workgroup gives the same results by index compare alone, with the code
