@@ -236,10 +236,11 @@ hipError_t launch_mask_colbits(const FaArgs& a, const uint8_t* flags, uint32_t* 
 // from the waves every entry would be four 4-byte stores from four places; instead the words cross LDS and every
 // thread stores complete entries, consecutive threads consecutive entries.  cw[e]: bit r = row r of the wave's 32;
 // key_of(lane, e): the key of a lane's e-th word.  (One spare entry after every sixteen keeps the word stores of a
-// wave on different banks.)
+// wave on different banks.)  `flags`: the class row of the attention mask for these query rows, or null: entries of
+// key blocks classed 'skip' are never read and are not written.
 template <typename KeyOf>
 ACCT_DEV void store_col_entries(uint32_t* s_cw, const uint32_t (&cw)[16], int wave, int lane, int key0, int Sk, uint32_t* out,
-                                KeyOf key_of) {
+                                const uint8_t* flags, KeyOf key_of) {
 #pragma unroll
   for (int e = 0; e < 16; e++) {
     const int k = key_of(lane, e);                       // 0 .. 1023 within the span
@@ -249,7 +250,7 @@ ACCT_DEV void store_col_entries(uint32_t* s_cw, const uint32_t (&cw)[16], int wa
 #pragma unroll
   for (int m = 0; m < 4; m++) {
     const int k = threadIdx.x + 256 * m;
-    if (key0 + k < Sk)
+    if (key0 + k < Sk && !(flags && flags[(key0 + k) >> 7] == kBlkSkip))
       *reinterpret_cast<u32x4*>(out + (int64_t)(key0 + k) * 4) = *reinterpret_cast<const u32x4*>(s_cw + (k + (k >> 4)) * 4);
   }
 }
@@ -335,7 +336,7 @@ __global__ void __launch_bounds__(256) fa_drop_bits_kernel(const FaArgs a, uint3
         uint32_t x = ((nz >> (KH * h)) & ((1u << KH) - 1u)) << (KH * (lane % LPW));
         x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xf, 0xf, true);                   // lane ^ 1
         if (LPW == 4) x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xf, 0xf, true);     // lane ^ 2
-        if (writer && rr < nrow && widx + 16 * h < a.droprow_w) rowout[16 * h] = x;
+        if (writer && rr < nrow && !dead[h] && widx + 16 * h < a.droprow_w) rowout[16 * h] = x;   // (words of hidden key blocks are never read)
       }
       rowout += a.droprow_w;
     }
@@ -359,7 +360,7 @@ __global__ void __launch_bounds__(256) fa_drop_bits_kernel(const FaArgs a, uint3
     }
   }
   if (colbits)
-    store_col_entries(s_cw, cw, i, lane, span * 1024, a.Sk, colbits + ((int64_t)bh * a.Tr + qb) * a.Sk * 4,
+    store_col_entries(s_cw, cw, i, lane, span * 1024, a.Sk, colbits + ((int64_t)bh * a.Tr + qb) * a.Sk * 4, flags,
                       [](int l, int e) { return ES == 1 ? 16 * l + e : 512 * (e >> 3) + 8 * l + (e & 7); });
 }
 
@@ -405,7 +406,7 @@ __global__ void __launch_bounds__(256) fa_drop_philox_kernel(const FaArgs a, uin
   if (colbits) {
 #pragma unroll
     for (int t = 0; t < 16; t++) cw[t] = __builtin_bitreverse32(cw[t]);
-    store_col_entries(s_cw, cw, i, lane, span * 1024, a.Sk, colbits + ((int64_t)bh * a.Tr + qb) * a.Sk * 4,
+    store_col_entries(s_cw, cw, i, lane, span * 1024, a.Sk, colbits + ((int64_t)bh * a.Tr + qb) * a.Sk * 4, nullptr,
                       [](int l, int t) { return 32 * (l >> 1) + 8 * (t >> 2) + 4 * (l & 1) + (t & 3); });
   }
 }
